@@ -1,0 +1,915 @@
+#include "engine.h"
+
+#include <string.h>
+#include <unistd.h>
+
+#include <algorithm>
+#include <chrono>
+
+#include "ipc.h"
+#include "log.h"
+#include "vmm.h"
+
+namespace amem {
+
+using Clock = std::chrono::steady_clock;
+static inline double ms_since(Clock::time_point t0) {
+  return std::chrono::duration<double, std::milli>(Clock::now() - t0).count();
+}
+
+Options& options() {
+  static Options o;
+  return o;
+}
+
+hipError_t DevBuf::ensure(size_t bytes) {
+  if (bytes <= cap) return hipSuccess;
+  release();
+  size_t want = std::max<size_t>(bytes + bytes / 4, 4096);
+  hipError_t e = CHECK_HIP(hipMalloc(&p, want));
+  if (e != hipSuccess) { p = nullptr; return e; }
+  cap = want;
+  return hipSuccess;
+}
+void DevBuf::release() {
+  if (p) (void)CHECK_HIP(hipFree(p));
+  p = nullptr;
+  cap = 0;
+}
+hipError_t PinBuf::ensure(size_t bytes) {
+  if (bytes <= cap) return hipSuccess;
+  release();
+  size_t want = std::max<size_t>(bytes + bytes / 4, 4096);
+  hipError_t e = CHECK_HIP(hipHostMalloc(&p, want, hipHostMallocDefault));
+  if (e != hipSuccess) { p = nullptr; return e; }
+  cap = want;
+  return hipSuccess;
+}
+void PinBuf::release() {
+  if (p) (void)CHECK_HIP(hipHostFree(p));
+  p = nullptr;
+  cap = 0;
+}
+
+Engine::Engine(int dev) : dev_(dev) {}
+
+Engine::~Engine() {
+  for (hipEvent_t e : events_) (void)hipEventDestroy(e);
+  DevBuf* db[] = {&d_segs_, &d_prefix_, &d_flags_, &d_sums_, &d_descs_, &d_tiles_, &d_slabtab_,
+                  &d_staging_[0], &d_staging_[1]};
+  for (DevBuf* b : db) b->release();
+  PinBuf* pb[] = {&h_segs_, &h_prefix_, &h_flags_, &h_sums_, &h_descs_, &h_tiles_, &h_slabtab_,
+                  &h_sums_verify_};
+  for (PinBuf* b : pb) b->release();
+  delete pool_;
+  if (kstream_) (void)hipStreamDestroy(kstream_);
+  if (dstream_) (void)hipStreamDestroy(dstream_);
+}
+
+hipError_t Engine::init() {
+  if (inited_) return hipSuccess;
+  hipError_t e = CHECK_HIP(hipSetDevice(dev_));
+  if (e != hipSuccess) return e;
+  // Non-blocking streams at the default priority: the null stream (on which the runtime
+  // runs map/unmap commands) must not wait for copies in flight.
+  e = CHECK_HIP(hipStreamCreateWithFlags(&kstream_, hipStreamNonBlocking));
+  if (e != hipSuccess) return e;
+  e = CHECK_HIP(hipStreamCreateWithFlags(&dstream_, hipStreamNonBlocking));
+  if (e != hipSuccess) return e;
+  pool_ = new SlabPool((uint64_t)options().slab_bytes);
+  inited_ = true;
+  return hipSuccess;
+}
+
+hipEvent_t Engine::event_at(size_t i) {
+  while (events_.size() <= i) {
+    hipEvent_t ev = nullptr;
+    (void)CHECK_HIP(hipEventCreate(&ev));
+    events_.push_back(ev);
+  }
+  return events_[i];
+}
+
+uint64_t Engine::trim_pool() {
+  if (!pool_) return 0;
+  slab_table_count_ = 0;
+  return pool_->trim();
+}
+
+// ---------------------------------------------------------------------------------------
+// scan
+// ---------------------------------------------------------------------------------------
+
+static uint64_t chunks_of(uint64_t bytes) { return (bytes + kChunkBytes - 1) / kChunkBytes; }
+
+hipError_t Engine::run_scan(const std::vector<ScanSeg>& segs, uint64_t* nchunks_out, bool want_sums,
+                            float* ms) {
+  const size_t n = segs.size();
+  hipError_t e;
+  if ((e = h_segs_.ensure(n * sizeof(ScanSeg))) != hipSuccess) return e;
+  if ((e = h_prefix_.ensure((n + 1) * sizeof(uint64_t))) != hipSuccess) return e;
+  uint64_t* prefix = (uint64_t*)h_prefix_.p;
+  uint64_t total = 0;
+  for (size_t i = 0; i < n; ++i) {
+    ((ScanSeg*)h_segs_.p)[i] = segs[i];
+    prefix[i] = total;
+    total += chunks_of(segs[i].bytes);
+  }
+  prefix[n] = total;
+  *nchunks_out = total;
+  if (total == 0) { if (ms) *ms = 0; return hipSuccess; }
+  if ((e = d_segs_.ensure(n * sizeof(ScanSeg))) != hipSuccess) return e;
+  if ((e = d_prefix_.ensure((n + 1) * sizeof(uint64_t))) != hipSuccess) return e;
+  if ((e = d_flags_.ensure(total)) != hipSuccess) return e;
+  if ((e = h_flags_.ensure(total)) != hipSuccess) return e;
+  if (want_sums) {
+    if ((e = d_sums_.ensure(total * sizeof(ChunkSum))) != hipSuccess) return e;
+  }
+  e = CHECK_HIP(hipMemcpyAsync(d_segs_.p, h_segs_.p, n * sizeof(ScanSeg), hipMemcpyHostToDevice, kstream_));
+  if (e != hipSuccess) return e;
+  e = CHECK_HIP(hipMemcpyAsync(d_prefix_.p, h_prefix_.p, (n + 1) * sizeof(uint64_t), hipMemcpyHostToDevice, kstream_));
+  if (e != hipSuccess) return e;
+  hipEvent_t e0 = event_at(0), e1 = event_at(1);
+  (void)CHECK_HIP(hipEventRecord(e0, kstream_));
+  e = CHECK_HIP(launch_scan((const ScanSeg*)d_segs_.p, (const uint64_t*)d_prefix_.p, (uint32_t)n, total,
+                            (uint8_t*)d_flags_.p, want_sums ? (ChunkSum*)d_sums_.p : nullptr,
+                            (uint32_t)options().hbm_wgs, kstream_));
+  if (e != hipSuccess) return e;
+  (void)CHECK_HIP(hipEventRecord(e1, kstream_));
+  e = CHECK_HIP(hipMemcpyAsync(h_flags_.p, d_flags_.p, total, hipMemcpyDeviceToHost, kstream_));
+  if (e != hipSuccess) return e;
+  e = CHECK_HIP(hipStreamSynchronize(kstream_));
+  if (e != hipSuccess) return e;
+  if (ms) {
+    *ms = 0;
+    (void)CHECK_HIP(hipEventElapsedTime(ms, e0, e1));
+  }
+  return hipSuccess;
+}
+
+hipError_t Engine::zero_scan(const amem_extent* ext, uint64_t n, uint8_t* flags, amem_chunk_sum* sums,
+                             float* ms) {
+  hipError_t e = init();
+  if (e != hipSuccess) return e;
+  std::vector<ScanSeg> segs(n);
+  for (uint64_t i = 0; i < n; ++i) {
+    if ((ext[i].va & 15) || (ext[i].bytes & 15) || ext[i].va == 0) return hipErrorInvalidValue;
+    segs[i] = {ext[i].va, ext[i].bytes};
+  }
+  uint64_t total = 0;
+  e = run_scan(segs, &total, sums != nullptr, ms);
+  if (e != hipSuccess || total == 0) return e;
+  memcpy(flags, h_flags_.p, total);
+  if (sums) {
+    e = CHECK_HIP(hipMemcpy(sums, d_sums_.p, total * sizeof(ChunkSum), hipMemcpyDeviceToHost));
+  }
+  return e;
+}
+
+// ---------------------------------------------------------------------------------------
+// descriptor plumbing
+// ---------------------------------------------------------------------------------------
+
+hipError_t Engine::upload_descs(const CopyDesc* descs, size_t n, uint64_t* ntiles_out) {
+  hipError_t e;
+  if ((e = h_descs_.ensure(std::max<size_t>(n, 1) * sizeof(CopyDesc))) != hipSuccess) return e;
+  if ((e = h_tiles_.ensure((n + 1) * sizeof(uint64_t))) != hipSuccess) return e;
+  if ((e = d_descs_.ensure(std::max<size_t>(n, 1) * sizeof(CopyDesc))) != hipSuccess) return e;
+  if ((e = d_tiles_.ensure((n + 1) * sizeof(uint64_t))) != hipSuccess) return e;
+  uint64_t* tp = (uint64_t*)h_tiles_.p;
+  uint64_t tiles = 0;
+  for (size_t i = 0; i < n; ++i) {
+    tp[i] = tiles;
+    tiles += (descs[i].bytes + kTileBytes - 1) / kTileBytes;
+  }
+  tp[n] = tiles;
+  *ntiles_out = tiles;
+  if (n) memcpy(h_descs_.p, descs, n * sizeof(CopyDesc));
+  if (n) {
+    e = CHECK_HIP(hipMemcpyAsync(d_descs_.p, h_descs_.p, n * sizeof(CopyDesc), hipMemcpyHostToDevice, kstream_));
+    if (e != hipSuccess) return e;
+  }
+  return CHECK_HIP(hipMemcpyAsync(d_tiles_.p, h_tiles_.p, (n + 1) * sizeof(uint64_t), hipMemcpyHostToDevice, kstream_));
+}
+
+// Device-side table of contiguous-side base addresses: pool slabs first, then the two
+// staging buffers, then one spare entry for the standalone entry points.
+hipError_t Engine::upload_slab_table() {
+  const size_t ns = pool_->slab_count();
+  const size_t entries = ns + 3;
+  hipError_t e;
+  if ((e = h_slabtab_.ensure(entries * sizeof(void*))) != hipSuccess) return e;
+  if ((e = d_slabtab_.ensure(entries * sizeof(void*))) != hipSuccess) return e;
+  uint8_t** tab = (uint8_t**)h_slabtab_.p;
+  for (size_t i = 0; i < ns; ++i) {
+    void* dp = nullptr;
+    e = CHECK_HIP(hipHostGetDevicePointer(&dp, pool_->slabs()[i], 0));
+    if (e != hipSuccess) return e;
+    tab[i] = (uint8_t*)dp;
+  }
+  tab[ns] = (uint8_t*)d_staging_[0].p;
+  tab[ns + 1] = (uint8_t*)d_staging_[1].p;
+  tab[ns + 2] = nullptr;
+  slab_table_count_ = ns;
+  return CHECK_HIP(hipMemcpyAsync(d_slabtab_.p, h_slabtab_.p, entries * sizeof(void*), hipMemcpyHostToDevice, kstream_));
+}
+
+// Append `d`, cut where its contiguous side would cross a slab boundary.
+static void push_split(std::vector<CopyDesc>& out, CopyDesc d, uint64_t slab_bytes) {
+  while (d.bytes) {
+    const uint64_t room = slab_bytes - (d.off & (slab_bytes - 1));
+    const uint64_t take = std::min(room, d.bytes);
+    out.push_back({d.va, d.off, take});
+    d.va += take; d.off += take; d.bytes -= take;
+  }
+}
+
+// Walk the chunks of one region and emit its runs. Non-zero runs take consecutive logical
+// offsets from *cursor; zero runs are emitted only when `zero_out` is given.
+static void emit_runs(const uint8_t* flags, uint64_t va, uint64_t size, bool elide, uint64_t* cursor,
+                      uint64_t slab_bytes, std::vector<CopyDesc>* data_out,
+                      std::vector<CopyDesc>* zero_out, uint64_t* zero_chunks) {
+  const uint64_t n = chunks_of(size);
+  uint64_t k = 0;
+  while (k < n) {
+    const bool z = elide && flags[k];
+    uint64_t j = k + 1;
+    while (j < n && (elide && flags[j]) == z) ++j;
+    const uint64_t start = k * kChunkBytes;
+    const uint64_t end = std::min(size, j * kChunkBytes);
+    if (z) {
+      if (zero_chunks) *zero_chunks += j - k;
+      if (zero_out) zero_out->push_back({va + start, kDescZero, end - start});
+    } else {
+      if (data_out) push_split(*data_out, {va + start, *cursor, end - start}, slab_bytes);
+      *cursor += end - start;
+    }
+    k = j;
+  }
+}
+
+hipError_t Engine::move(bool scatter, const amem_copy_desc* descs, uint64_t n, void* staging,
+                        uint64_t staging_bytes, bool host_side, float* ms) {
+  hipError_t e = init();
+  if (e != hipSuccess) return e;
+  if (ms) *ms = 0;
+  if (n == 0) return hipSuccess;
+  if (!staging || ((uintptr_t)staging & 15)) return hipErrorInvalidValue;
+  std::vector<CopyDesc> v(n);
+  for (uint64_t i = 0; i < n; ++i) {
+    const amem_copy_desc& d = descs[i];
+    if (d.va == 0 || (d.va & 15) || (d.bytes & 15)) return hipErrorInvalidValue;
+    if (d.off == kDescZero) {
+      if (!scatter) return hipErrorInvalidValue;
+    } else if ((d.off & 15) || d.off > staging_bytes || d.bytes > staging_bytes - d.off) {
+      return hipErrorInvalidValue;
+    }
+    v[i] = {d.va, d.off, d.bytes};
+  }
+  uint64_t ntiles = 0;
+  if ((e = upload_descs(v.data(), v.size(), &ntiles)) != hipSuccess) return e;
+  if (slab_table_count_ != pool_->slab_count() || !d_slabtab_.p) {
+    if ((e = upload_slab_table()) != hipSuccess) return e;
+  }
+  void* dp = staging;
+  if (host_side) {
+    e = CHECK_HIP(hipHostGetDevicePointer(&dp, staging, 0));
+    if (e != hipSuccess) return e;
+  }
+  const size_t spare = pool_->slab_count() + 2;
+  ((uint8_t**)h_slabtab_.p)[spare] = (uint8_t*)dp;
+  e = CHECK_HIP(hipMemcpyAsync((uint8_t**)d_slabtab_.p + spare, (uint8_t**)h_slabtab_.p + spare,
+                               sizeof(void*), hipMemcpyHostToDevice, kstream_));
+  if (e != hipSuccess) return e;
+  SlabTable st = {(uint8_t* const*)d_slabtab_.p + spare, 63, ~(uint64_t)0 >> 1};
+  hipEvent_t e0 = event_at(0), e1 = event_at(1);
+  (void)CHECK_HIP(hipEventRecord(e0, kstream_));
+  e = CHECK_HIP(launch_move(scatter, (const CopyDesc*)d_descs_.p, (const uint64_t*)d_tiles_.p,
+                            (uint32_t)n, 0, ntiles, st, 0,
+                            (uint32_t)(host_side ? options().link_wgs : options().hbm_wgs), kstream_));
+  if (e != hipSuccess) return e;
+  (void)CHECK_HIP(hipEventRecord(e1, kstream_));
+  e = CHECK_HIP(hipStreamSynchronize(kstream_));
+  if (e == hipSuccess && ms) (void)CHECK_HIP(hipEventElapsedTime(ms, e0, e1));
+  return e;
+}
+
+// ---------------------------------------------------------------------------------------
+// pause
+// ---------------------------------------------------------------------------------------
+
+static int popcount_peers(const Region& r) {
+  int n = 0;
+  for (int i = 0; i < AMEM_MAX_DEVS; ++i) n += (r.peers[i] != 0);
+  return n;
+}
+
+// Reference step 3 for one region (amem_nccl.cpp:529-557): drop the mapping and every
+// reference, mark HOLE, forget the handle.
+hipError_t Engine::release_local(Ctx& c, Region* r, uint64_t va) {
+  auto t0 = Clock::now();
+  uint64_t old = r->handle ? r->handle : vmm_handle_of(va);
+  if (r->type == AMEM_TYPE_LOCAL_SYMM)
+    LOGGER(DEBUG, "memPause: dptr:%llx is symmetric memory; no multicast object to unbind on this platform",
+           (unsigned long long)va);
+  if (r->refcount > 0)
+    LOGGER(DEBUG, "memPause: groupID:%d pid:%d dptr:%llx refcount:%d", amem_groupID_value(), getpid(),
+           (unsigned long long)va, r->refcount);
+  hipError_t e = vmm_unmap_release(va, r->allocSz, old, r->refcount);
+  {
+    std::lock_guard<std::mutex> lk(c.fields);
+    c.releaseLocalCnt += popcount_peers(*r);
+    r->state = AMEM_STATE_HOLE;
+    r->handle = 0;
+  }
+  c.handleTable[dev_].erase(old);
+  stats_.pause_unmap_ms += ms_since(t0);
+  return e;
+}
+
+// Direct path: one gather kernel writes pinned host memory; runs of at least
+// dma_min_bytes go by hipMemcpyAsync on the second stream at the same time.
+hipError_t Engine::pause_copy_direct(Ctx& c, std::vector<Region*>& regs) {
+  hipError_t e = hipSuccess;
+  const uint64_t dma_min = (uint64_t)options().dma_min_bytes;
+  std::vector<CopyDesc> kdescs;
+  kdescs.reserve(gather_descs_.size());
+  auto tc = Clock::now();
+  for (const CopyDesc& d : gather_descs_) {
+    if (dma_min && d.bytes >= dma_min) {
+      e = CHECK_HIP(hipMemcpyAsync(pool_->host_addr(d.off), (const void*)(uintptr_t)d.va, d.bytes,
+                                   hipMemcpyDeviceToHost, dstream_));
+      if (e != hipSuccess) return e;
+      stats_.dma_bytes += d.bytes;
+    } else {
+      kdescs.push_back(d);
+      stats_.kernel_bytes += d.bytes;
+    }
+  }
+  uint64_t ntiles = 0;
+  if ((e = upload_descs(kdescs.data(), kdescs.size(), &ntiles)) != hipSuccess) return e;
+  SlabTable st = {(uint8_t* const*)d_slabtab_.p, pool_->shift(), pool_->slab_bytes() - 1};
+  hipEvent_t e0 = event_at(4), e1 = event_at(5);
+  (void)CHECK_HIP(hipEventRecord(e0, kstream_));
+  e = CHECK_HIP(launch_move(false, (const CopyDesc*)d_descs_.p, (const uint64_t*)d_tiles_.p,
+                            (uint32_t)kdescs.size(), 0, ntiles, st, 0, (uint32_t)options().link_wgs, kstream_));
+  if (e != hipSuccess) return e;
+  (void)CHECK_HIP(hipEventRecord(e1, kstream_));
+  if (ntiles) stats_.k2_launches++;
+  e = CHECK_HIP(hipStreamSynchronize(kstream_));
+  if (e != hipSuccess) return e;
+  e = CHECK_HIP(hipStreamSynchronize(dstream_));
+  if (e != hipSuccess) return e;
+  stats_.pause_copy_ms = ms_since(tc);
+  float ms = 0;
+  if (ntiles && hipEventElapsedTime(&ms, e0, e1) == hipSuccess) stats_.k2_ms += ms;
+  for (size_t i = 0; i < regs.size(); ++i) {
+    hipError_t e2 = release_local(c, regs[i], parked_[i].va);
+    if (e == hipSuccess) e = e2;
+  }
+  return e;
+}
+
+// Staged path: regions are taken in rounds that fit one device staging buffer. A round is
+// packed by a gather kernel at HBM rate, then leaves as a few large hipMemcpyAsync calls
+// while the host unmaps and releases that round's regions. No kernel is in flight while
+// the host unmaps: an unmap issued under a running kernel stalls for milliseconds, one
+// issued under a copy-engine transfer does not.
+hipError_t Engine::pause_copy_staged(Ctx& c, std::vector<Region*>& regs, bool* used) {
+  *used = false;
+  const uint64_t cap = (uint64_t)options().staging_bytes;
+  if (cap < kChunkBytes) return hipSuccess;
+  const uint64_t need = std::min<uint64_t>(cap, std::max<uint64_t>(parked_total_, kChunkBytes));
+  for (int b = 0; b < 2; ++b) {
+    if (d_staging_[b].cap >= need) continue;
+    d_staging_[b].release();
+    void* p = nullptr;
+    if (hipMalloc(&p, need) != hipSuccess) {
+      (void)hipGetLastError();
+      LOGGER(INFO, "memPause: no room for %llu MiB of device staging, using the direct path",
+             (unsigned long long)(need >> 20));
+      d_staging_[0].release();
+      d_staging_[1].release();
+      return hipSuccess;
+    }
+    d_staging_[b].p = p;
+    d_staging_[b].cap = need;
+  }
+  *used = true;
+  hipError_t e;
+  uint64_t ntiles_all = 0;
+  if ((e = upload_descs(gather_descs_.data(), gather_descs_.size(), &ntiles_all)) != hipSuccess) return e;
+  if ((e = upload_slab_table()) != hipSuccess) return e;
+  const uint64_t* tp = (const uint64_t*)h_tiles_.p;
+  const size_t ns = pool_->slab_count();
+  SlabTable pool_tab = {(uint8_t* const*)d_slabtab_.p, pool_->shift(), pool_->slab_bytes() - 1};
+  auto tc = Clock::now();
+  size_t ev = 8;  // events 8.. are per-launch timing pairs
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> timed;
+  hipEvent_t dma_done[2] = {event_at(2), event_at(3)};
+  bool dma_pending[2] = {false, false};
+  size_t i = 0;
+  int round = 0;
+  const size_t n = parked_.size();
+  const uint64_t room = d_staging_[0].cap;
+  while (i < n) {
+    // a round: regions [i, j), descriptors [d0, d1), logical offsets [base, base + bytes)
+    size_t j = i;
+    uint64_t bytes = 0;
+    const bool big = parked_[i].parked_bytes > room;
+    if (big) { bytes = parked_[i].parked_bytes; j = i + 1; }
+    else while (j < n && bytes + parked_[j].parked_bytes <= room) bytes += parked_[j++].parked_bytes;
+    const uint32_t d0 = parked_[i].desc_begin, d1 = parked_[j - 1].desc_end;
+    const uint64_t base = parked_[i].parked_off;
+    const int buf = round & 1;
+    if (bytes) {
+      hipEvent_t s0 = event_at(ev++), s1 = event_at(ev++);
+      if (big) {
+        // larger than a staging buffer: straight to host memory
+        (void)CHECK_HIP(hipEventRecord(s0, kstream_));
+        e = CHECK_HIP(launch_move(false, (const CopyDesc*)d_descs_.p + d0, (const uint64_t*)d_tiles_.p + d0,
+                                  d1 - d0, tp[d0], tp[d1] - tp[d0], pool_tab, 0,
+                                  (uint32_t)options().link_wgs, kstream_));
+        if (e != hipSuccess) return e;
+        (void)CHECK_HIP(hipEventRecord(s1, kstream_));
+        e = CHECK_HIP(hipEventSynchronize(s1));
+        if (e != hipSuccess) return e;
+        stats_.kernel_bytes += bytes;
+      } else {
+        if (dma_pending[buf]) {
+          e = CHECK_HIP(hipEventSynchronize(dma_done[buf]));
+          if (e != hipSuccess) return e;
+          dma_pending[buf] = false;
+        }
+        SlabTable stg = {(uint8_t* const*)d_slabtab_.p + ns + buf, 63, ~(uint64_t)0 >> 1};
+        (void)CHECK_HIP(hipEventRecord(s0, kstream_));
+        e = CHECK_HIP(launch_move(false, (const CopyDesc*)d_descs_.p + d0, (const uint64_t*)d_tiles_.p + d0,
+                                  d1 - d0, tp[d0], tp[d1] - tp[d0], stg, base,
+                                  (uint32_t)options().hbm_wgs, kstream_));
+        if (e != hipSuccess) return e;
+        (void)CHECK_HIP(hipEventRecord(s1, kstream_));
+        e = CHECK_HIP(hipEventSynchronize(s1));
+        if (e != hipSuccess) return e;
+        uint64_t x = 0;
+        while (x < bytes) {
+          const uint64_t take = std::min(bytes - x, pool_->room(base + x));
+          e = CHECK_HIP(hipMemcpyAsync(pool_->host_addr(base + x), (uint8_t*)d_staging_[buf].p + x, take,
+                                       hipMemcpyDeviceToHost, dstream_));
+          if (e != hipSuccess) return e;
+          x += take;
+        }
+        (void)CHECK_HIP(hipEventRecord(dma_done[buf], dstream_));
+        dma_pending[buf] = true;
+        stats_.dma_bytes += bytes;
+      }
+      timed.push_back({s0, s1});
+      stats_.k2_launches++;
+      ++round;
+    }
+    for (size_t r = i; r < j; ++r) {
+      hipError_t e2 = release_local(c, regs[r], parked_[r].va);
+      if (e2 != hipSuccess) return e2;
+    }
+    i = j;
+  }
+  e = CHECK_HIP(hipStreamSynchronize(dstream_));
+  if (e != hipSuccess) return e;
+  stats_.pause_copy_ms = ms_since(tc);
+  for (auto& pr : timed) {
+    float ms = 0;
+    if (hipEventElapsedTime(&ms, pr.first, pr.second) == hipSuccess) stats_.k2_ms += ms;
+  }
+  // Device staging is given back: a paused process should hold no device memory for this.
+  d_staging_[0].release();
+  d_staging_[1].release();
+  return hipSuccess;
+}
+
+int Engine::pause(Ctx& c) {
+  auto t0 = Clock::now();
+  hipError_t e = init();
+  if (e != hipSuccess) return (int)e;
+  int rc = 0;
+  auto note = [&](hipError_t x) { if (x != hipSuccess && rc == 0) rc = (int)x; };
+  const bool elide = options().zero_elide != 0;
+  amem_cycle_stats fresh = {};
+  fresh.slab_bytes = stats_.slab_bytes;
+  stats_ = fresh;
+
+  auto& table = c.allocTable[dev_];
+  note(CHECK_HIP(hipDeviceSynchronize()));
+  size_t free_sz = 0, total = 0;
+  (void)CHECK_HIP(hipMemGetInfo(&free_sz, &total));
+  LOGGER(INFO, "memPause: groupID:%d pid:%d GPU:%d memUsed: %ld MB before paused", amem_groupID_value(),
+         getpid(), dev_, (long)((total - free_sz) >> 20));
+
+  std::vector<Region*> locals;
+  std::vector<std::pair<uint64_t, Region*>> imported;
+  parked_.clear();
+  gather_descs_.clear();
+  segs_.clear();
+  for (auto& kv : table) {
+    Region& r = kv.second;
+    if (r.state != AMEM_STATE_ALLOC) continue;
+    if (from_peer(r.type)) imported.push_back({kv.first, &r});
+    else {
+      locals.push_back(&r);
+      segs_.push_back({kv.first, (uint64_t)r.allocSz});
+    }
+  }
+
+  // Imported mappings go first (reference step 2, amem_nccl.cpp:517-526): no data to save,
+  // and the owner's release only frees memory once importers have let go.
+  for (auto& pr : imported) {
+    auto tu = Clock::now();
+    Region* r = pr.second;
+    LOGGER(DEBUG, "memPause: release peer handle %llx.", (unsigned long long)pr.first);
+    uint64_t h = r->handle ? r->handle : vmm_handle_of(pr.first);
+    note(vmm_unmap_release(pr.first, r->allocSz, h, 0));
+    std::lock_guard<std::mutex> lk(c.fields);
+    r->state = AMEM_STATE_HOLE;
+    c.releaseShadowCnt++;
+    stats_.pause_unmap_ms += ms_since(tu);
+  }
+  stats_.peer_regions = imported.size();
+  stats_.local_regions = locals.size();
+
+  // Reference step 1 (amem_nccl.cpp:502-513): save the bytes of every local region.
+  {
+    std::lock_guard<std::mutex> lk(c.fields);
+    for (Region* r : locals) { r->state = AMEM_STATE_OFFLOADING; c.offloadCnt++; }
+  }
+  auto ts = Clock::now();
+  float k1ms = 0;
+  have_sums_ = true;
+  e = run_scan(segs_, &nchunks_, true, &k1ms);
+  note(e);
+  if (e == hipSuccess && nchunks_) {
+    note(h_sums_.ensure(nchunks_ * sizeof(ChunkSum)));
+    note(CHECK_HIP(hipMemcpyAsync(h_sums_.p, d_sums_.p, nchunks_ * sizeof(ChunkSum), hipMemcpyDeviceToHost, kstream_)));
+  }
+  stats_.k1_ms = k1ms;
+  stats_.k1_launches = nchunks_ ? 1 : 0;
+  stats_.pause_scan_ms = ms_since(ts);
+  stats_.total_chunks = nchunks_;
+
+  auto tp = Clock::now();
+  uint64_t cursor = 0, chunk0 = 0, zero_chunks = 0;
+  const uint8_t* flags = (const uint8_t*)h_flags_.p;
+  uint64_t slab_bytes = pool_->slab_bytes();
+  for (size_t i = 0; i < locals.size(); ++i) {
+    ParkedRegion p = {};
+    p.va = segs_[i].va;
+    p.size = segs_[i].bytes;
+    p.first_chunk = chunk0;
+    p.nchunks = chunks_of(p.size);
+    p.parked_off = cursor;
+    p.desc_begin = (uint32_t)gather_descs_.size();
+    emit_runs(flags + chunk0, p.va, p.size, elide, &cursor, slab_bytes, &gather_descs_, nullptr, &zero_chunks);
+    p.desc_end = (uint32_t)gather_descs_.size();
+    p.parked_bytes = cursor - p.parked_off;
+    chunk0 += p.nchunks;
+    stats_.footprint_bytes += p.size;
+    parked_.push_back(p);
+  }
+  parked_total_ = cursor;
+  stats_.parked_bytes = cursor;
+  stats_.zero_chunks = zero_chunks;
+  e = pool_->ensure(cursor);
+  note(e);
+  stats_.slab_bytes = pool_->capacity();
+  for (size_t i = 0; i < locals.size(); ++i) {
+    locals[i]->parkedBytes = parked_[i].parked_bytes;
+    locals[i]->cpuAddr = (parked_[i].parked_bytes && e == hipSuccess) ? pool_->host_addr(parked_[i].parked_off) : nullptr;
+  }
+  stats_.pause_plan_ms = ms_since(tp);
+
+  if (rc == 0) {
+    bool staged = false;
+    const int64_t path = options().pause_path;
+    if (path != 0 && !locals.empty()) note(pause_copy_staged(c, locals, &staged));
+    if (!staged && rc == 0) {
+      note(upload_slab_table());
+      note(pause_copy_direct(c, locals));
+    }
+  }
+  // The sums copy above rode kstream_; make sure it landed before the scratch is reused.
+  note(CHECK_HIP(hipStreamSynchronize(kstream_)));
+
+  // Reference step 3 also releases local regions that were not in ALLOC state and so were
+  // not saved (amem_nccl.cpp:529-557 has no state test).
+  if (rc == 0) {
+    for (auto& kv : table) {
+      Region& r = kv.second;
+      if (!from_peer(r.type) && r.state != AMEM_STATE_HOLE) note(release_local(c, &r, kv.first));
+    }
+  } else {
+    LOGGER(ERROR, "memPause: groupID:%d pid:%d GPU:%d failed with HIP error %d; physical memory of "
+           "regions not yet released stays mapped", amem_groupID_value(), getpid(), dev_, rc);
+  }
+  note(CHECK_HIP(hipStreamSynchronize(dstream_)));
+  c.pauseCnt++;
+  stats_.pause_ms = ms_since(t0);
+  (void)CHECK_HIP(hipMemGetInfo(&free_sz, &total));
+  LOGGER(INFO, "memPause: pause results. groupID:%d pid:%d GPU:%d pauseCnt:%ld memUsed:%ld MB after paused, "
+         "released:%ld MB, duration:%ld ms offload:%d releaseLocal:%d releasePeer:%d",
+         amem_groupID_value(), getpid(), dev_, (long)c.pauseCnt, (long)((total - free_sz) >> 20),
+         (long)(stats_.footprint_bytes >> 20), (long)stats_.pause_ms, c.offloadCnt, c.releaseLocalCnt,
+         c.releaseShadowCnt);
+  return rc;
+}
+
+void Engine::forget(uint64_t va) {
+  for (ParkedRegion& p : parked_) {
+    if (p.va == va) { p.va = 0; break; }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// resume
+// ---------------------------------------------------------------------------------------
+
+int Engine::resume(Ctx& c) {
+  hipError_t e = init();
+  if (e != hipSuccess) return (int)e;
+  int rc = 0;
+  auto note = [&](hipError_t x) { if (x != hipSuccess && rc == 0) rc = (int)x; };
+  const bool elide = options().zero_elide != 0;
+  size_t free_sz = 0, total = 0;
+  (void)CHECK_HIP(hipMemGetInfo(&free_sz, &total));
+  LOGGER(INFO, "groupID:%d pid:%d GPU:%d memUsed:%ld MB before resumed", amem_groupID_value(), getpid(), dev_,
+         (long)((total - free_sz) >> 20));
+  auto t0 = Clock::now();
+  stats_.resume_ms = stats_.resume_map_ms = stats_.resume_copy_ms = stats_.resume_peer_ms = 0;
+  stats_.k3_ms = 0; stats_.k3_launches = 0; stats_.verify_mismatch = 0;
+  auto& table = c.allocTable[dev_];
+
+  // Scatter list: per region, its parked runs and its zero runs.
+  struct Item { Region* r; uint64_t va; uint32_t d0, d1; uint64_t bytes; };
+  std::vector<Item> items;
+  std::vector<CopyDesc> scatter;
+  const uint8_t* flags = (const uint8_t*)h_flags_.p;
+  const uint64_t slab_bytes = pool_->slab_bytes();
+  std::vector<ScanSeg> verify_segs;
+  std::vector<uint64_t> verify_first_chunk;
+  for (const ParkedRegion& p : parked_) {
+    if (p.va == 0) continue;
+    auto it = table.find(p.va);
+    if (it == table.end()) continue;
+    Region& r = it->second;
+    if (r.state != AMEM_STATE_HOLE || from_peer(r.type)) continue;
+    Item im = {&r, p.va, (uint32_t)scatter.size(), 0, p.size};
+    uint64_t cursor = p.parked_off;
+    std::vector<CopyDesc> zeros;
+    emit_runs(flags + p.first_chunk, p.va, p.size, elide, &cursor, slab_bytes, &scatter, &zeros, nullptr);
+    scatter.insert(scatter.end(), zeros.begin(), zeros.end());
+    im.d1 = (uint32_t)scatter.size();
+    items.push_back(im);
+    verify_segs.push_back({p.va, p.size});
+    verify_first_chunk.push_back(p.first_chunk);
+  }
+  // Local holes that were never saved come back as zeros.
+  for (auto& kv : table) {
+    Region& r = kv.second;
+    if (r.state != AMEM_STATE_HOLE || from_peer(r.type)) continue;
+    bool known = false;
+    for (const Item& im : items) if (im.va == kv.first) { known = true; break; }
+    if (known) continue;
+    Item im = {&r, kv.first, (uint32_t)scatter.size(), 0, (uint64_t)r.allocSz};
+    scatter.push_back({kv.first, kDescZero, (uint64_t)r.allocSz & ~(uint64_t)15});
+    im.d1 = (uint32_t)scatter.size();
+    items.push_back(im);
+  }
+  uint64_t ntiles_all = 0;
+  note(upload_descs(scatter.data(), scatter.size(), &ntiles_all));
+  note(upload_slab_table());
+  const uint64_t* tp = (const uint64_t*)h_tiles_.p;
+  SlabTable pool_tab = {(uint8_t* const*)d_slabtab_.p, pool_->shift(), pool_->slab_bytes() - 1};
+
+  struct Export { Region* r; uint64_t va; int fd; };
+  std::vector<Export> exports;
+  uint64_t exportSz = 0;
+  size_t ev = 8;
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> timed;
+  auto tc = Clock::now();
+  const uint64_t batch_bytes = (uint64_t)std::max<int64_t>(options().resume_batch_bytes, 1);
+  size_t i = 0;
+  while (i < items.size() && rc == 0) {
+    size_t j = i;
+    uint64_t bytes = 0;
+    auto tm = Clock::now();
+    while (j < items.size() && (bytes < batch_bytes || j == i)) {
+      Item& im = items[j];
+      uint64_t newh = 0;
+      // amem_cuAllocAndExport (amem_nccl.h:164-193): create, map at the same VA, grant access.
+      e = vmm_create_map(im.va, dev_, im.r->allocSz, &newh);
+      note(e);
+      if (e != hipSuccess) break;
+      if (im.r->type == AMEM_TYPE_LOCAL_SYMM)
+        LOGGER(DEBUG, "memResume: dptr:%llx is symmetric memory; no multicast object to bind on this platform",
+               (unsigned long long)im.va);
+      bool has_peer;
+      {
+        std::lock_guard<std::mutex> lk(c.fields);
+        im.r->state = AMEM_STATE_PRELOADING;
+        im.r->handle = newh;  // amem_updateAllocInfo, amem_nccl.cpp:272-291
+        im.r->handleGen++;
+        has_peer = im.r->hasPeer;
+      }
+      if (has_peer) {
+        int fd = -1;
+        note(vmm_export_fd(newh, &fd));
+        exports.push_back({im.r, im.va, fd});
+        exportSz += im.r->allocSz;
+      }
+      c.handleTable[dev_].emplace(newh, im.va);
+      bytes += im.bytes;
+      ++j;
+    }
+    stats_.resume_map_ms += ms_since(tm);
+    if (j == i) break;
+    const uint32_t d0 = items[i].d0, d1 = items[j - 1].d1;
+    if (d1 > d0 && tp[d1] > tp[d0]) {
+      hipEvent_t s0 = event_at(ev++), s1 = event_at(ev++);
+      (void)CHECK_HIP(hipEventRecord(s0, kstream_));
+      note(CHECK_HIP(launch_move(true, (const CopyDesc*)d_descs_.p + d0, (const uint64_t*)d_tiles_.p + d0,
+                                 d1 - d0, tp[d0], tp[d1] - tp[d0], pool_tab, 0,
+                                 (uint32_t)options().link_wgs, kstream_)));
+      (void)CHECK_HIP(hipEventRecord(s1, kstream_));
+      timed.push_back({s0, s1});
+      stats_.k3_launches++;
+    }
+    {
+      std::lock_guard<std::mutex> lk(c.fields);
+      for (size_t k = i; k < j; ++k) { items[k].r->state = AMEM_STATE_ALLOC; c.offloadCnt--; }
+    }
+    i = j;
+  }
+  note(CHECK_HIP(hipStreamSynchronize(kstream_)));
+  stats_.resume_copy_ms = ms_since(tc);
+  for (auto& pr : timed) {
+    float ms = 0;
+    if (hipEventElapsedTime(&ms, pr.first, pr.second) == hipSuccess) stats_.k3_ms += ms;
+  }
+
+  if (options().verify && have_sums_ && rc == 0 && !verify_segs.empty()) {
+    uint64_t nch = 0;
+    float ms = 0;
+    e = run_scan(verify_segs, &nch, true, &ms);
+    note(e);
+    if (e == hipSuccess) {
+      note(h_sums_verify_.ensure(nch * sizeof(ChunkSum)));
+      note(CHECK_HIP(hipMemcpy(h_sums_verify_.p, d_sums_.p, nch * sizeof(ChunkSum), hipMemcpyDeviceToHost)));
+      const ChunkSum* before = (const ChunkSum*)h_sums_.p;
+      const ChunkSum* after = (const ChunkSum*)h_sums_verify_.p;
+      uint64_t a = 0;
+      for (size_t s = 0; s < verify_segs.size(); ++s) {
+        const uint64_t n = chunks_of(verify_segs[s].bytes);
+        for (uint64_t k = 0; k < n; ++k, ++a) {
+          const ChunkSum& b = before[verify_first_chunk[s] + k];
+          if (b.sum64 != after[a].sum64 || b.xor64 != after[a].xor64) stats_.verify_mismatch++;
+        }
+      }
+      if (stats_.verify_mismatch) {
+        LOGGER(ERROR, "memResume: %llu chunks differ from their pre-pause checksum",
+               (unsigned long long)stats_.verify_mismatch);
+        if (rc == 0) rc = (int)hipErrorUnknown;
+      }
+    }
+  }
+
+  // Tell every importer where the new memory is (amem_nccl.cpp:633-649), after the bytes
+  // are back so that an importer never maps memory still being filled.
+  auto tpeer = Clock::now();
+  for (Export& x : exports) {
+    uint64_t peers[AMEM_MAX_DEVS];
+    {
+      std::lock_guard<std::mutex> lk(c.fields);
+      memcpy(peers, x.r->peers, sizeof(peers));
+    }
+    for (int s = 0; s < AMEM_MAX_DEVS; ++s) {
+      if (peers[s] == 0) continue;
+      int ret = peer_update(s, peers[s], x.fd);
+      if (ret != 0) {
+        LOGGER(ERROR, "groupID:%d pid:%d localDptr:%llx newHandle:%llx fd:%d notify peer %d to remap dptr:%llx ret:%d",
+               amem_groupID_value(), getpid(), (unsigned long long)x.va, (unsigned long long)x.r->handle, x.fd,
+               s, (unsigned long long)peers[s], ret);
+        if (rc == 0) rc = ret;
+      } else {
+        std::lock_guard<std::mutex> lk(c.fields);
+        c.releaseLocalCnt--;
+      }
+    }
+    if (x.fd >= 0) close(x.fd);
+  }
+
+  // Wait until every mapping this process imports has been re-established by its owner
+  // (amem_nccl.cpp:659-662 polls every 500 ms; here the service thread signals).
+  {
+    std::unique_lock<std::mutex> lk(c.fields);
+    const int64_t tmo = options().peer_timeout_ms;
+    auto done = [&] { return c.releaseShadowCnt <= 0; };
+    if (tmo > 0) {
+      if (!c.shadow_cv.wait_for(lk, std::chrono::milliseconds(tmo), done)) {
+        LOGGER(ERROR, "groupID:%d pid:%d GPU:%d peerLeft:%d after %lld ms, giving up", amem_groupID_value(),
+               getpid(), dev_, c.releaseShadowCnt, (long long)tmo);
+        if (rc == 0) rc = 1;
+      }
+    } else {
+      c.shadow_cv.wait(lk, done);
+    }
+  }
+  stats_.resume_peer_ms = ms_since(tpeer);
+  stats_.resume_ms = ms_since(t0);
+  (void)CHECK_HIP(hipMemGetInfo(&free_sz, &total));
+  LOGGER(INFO, "groupID:%d pid:%d GPU:%d resumeCnt:%ld memUsed:%ld MB after resumed, duration:%ld ms "
+         "offloadLeft:%d releaseLocalLeft:%d releasePeerLeft:%d exportSz:%ld",
+         amem_groupID_value(), getpid(), dev_, (long)(c.resumeCnt + 1), (long)((total - free_sz) >> 20),
+         (long)stats_.resume_ms, c.offloadCnt, c.releaseLocalCnt, c.releaseShadowCnt, (long)(exportSz >> 20));
+  return rc;
+}
+
+// ---------------------------------------------------------------------------------------
+// measurement helpers
+// ---------------------------------------------------------------------------------------
+
+hipError_t Engine::probe_link(uint64_t bytes, int reps, double* d2h, double* h2d) {
+  hipError_t e = init();
+  if (e != hipSuccess) return e;
+  void *hp = nullptr, *dp = nullptr;
+  if ((e = CHECK_HIP(hipHostMalloc(&hp, bytes, hipHostMallocDefault))) != hipSuccess) return e;
+  if ((e = CHECK_HIP(hipMalloc(&dp, bytes))) != hipSuccess) { (void)hipHostFree(hp); return e; }
+  memset(hp, 0x5a, bytes);
+  (void)CHECK_HIP(hipMemset(dp, 0xa5, bytes));
+  double best_d2h = 0, best_h2d = 0;
+  for (int r = 0; r < reps + 1 && e == hipSuccess; ++r) {
+    (void)CHECK_HIP(hipDeviceSynchronize());
+    auto t0 = Clock::now();
+    e = CHECK_HIP(hipMemcpy(hp, dp, bytes, hipMemcpyDeviceToHost));
+    double a = ms_since(t0);
+    t0 = Clock::now();
+    if (e == hipSuccess) e = CHECK_HIP(hipMemcpy(dp, hp, bytes, hipMemcpyHostToDevice));
+    double b = ms_since(t0);
+    if (r == 0) continue;  // first pass touches the pinned pages
+    best_d2h = std::max(best_d2h, bytes / a / 1e6);
+    best_h2d = std::max(best_h2d, bytes / b / 1e6);
+  }
+  (void)CHECK_HIP(hipFree(dp));
+  (void)CHECK_HIP(hipHostFree(hp));
+  if (d2h) *d2h = best_d2h;
+  if (h2d) *h2d = best_h2d;
+  return e;
+}
+
+hipError_t Engine::calib_copy(uint64_t bytes, int reps, float* ms) {
+  hipError_t e = init();
+  if (e != hipSuccess) return e;
+  bytes &= ~(uint64_t)15;
+  void *a = nullptr, *b = nullptr;
+  if ((e = CHECK_HIP(hipMalloc(&a, bytes))) != hipSuccess) return e;
+  if ((e = CHECK_HIP(hipMalloc(&b, bytes))) != hipSuccess) { (void)hipFree(a); return e; }
+  (void)CHECK_HIP(hipMemset(a, 0x11, bytes));
+  (void)CHECK_HIP(hipDeviceSynchronize());
+  hipEvent_t e0 = event_at(0), e1 = event_at(1);
+  float best = 0;
+  for (int r = 0; r < reps && e == hipSuccess; ++r) {
+    (void)CHECK_HIP(hipEventRecord(e0, kstream_));
+    e = CHECK_HIP(launch_calib_copy(a, b, bytes, kstream_));
+    (void)CHECK_HIP(hipEventRecord(e1, kstream_));
+    if (e == hipSuccess) e = CHECK_HIP(hipStreamSynchronize(kstream_));
+    float t = 0;
+    if (e == hipSuccess && hipEventElapsedTime(&t, e0, e1) == hipSuccess && (best == 0 || t < best)) best = t;
+  }
+  (void)CHECK_HIP(hipFree(a));
+  (void)CHECK_HIP(hipFree(b));
+  if (ms) *ms = best;
+  return e;
+}
+
+// ---------------------------------------------------------------------------------------
+// per-device singletons
+// ---------------------------------------------------------------------------------------
+
+static Engine* g_engines[AMEM_MAX_DEVS] = {nullptr};
+static std::mutex g_engines_mtx;
+
+Engine* engine_for(int dev) {
+  if (dev < 0 || dev >= AMEM_MAX_DEVS) return nullptr;
+  std::lock_guard<std::mutex> lk(g_engines_mtx);
+  if (g_engines[dev]) return g_engines[dev];
+  if (!gpu_present()) {
+    LOGGER(ERROR, "pid:%d no HIP device is visible: the pause/resume data path has no host fallback", getpid());
+    return nullptr;
+  }
+  Engine* en = new Engine(dev);
+  if (en->init() != hipSuccess) { delete en; return nullptr; }
+  g_engines[dev] = en;
+  return en;
+}
+
+void destroy_engines() {
+  std::lock_guard<std::mutex> lk(g_engines_mtx);
+  for (int i = 0; i < AMEM_MAX_DEVS; ++i) { delete g_engines[i]; g_engines[i] = nullptr; }
+}
+
+}  // namespace amem

@@ -1,0 +1,119 @@
+// The pause/resume data path on one GPU: zero/checksum scan, packing into pinned host
+// memory, physical release, and the reverse. Replaces the bodies of amem_memPause /
+// amem_memResume (amem_nccl_plugin/amem_nccl.cpp:467-677), whose data path is one
+// synchronous cuMemcpy per region.
+#ifndef AMEM_ENGINE_H_
+#define AMEM_ENGINE_H_
+
+#include <hip/hip_runtime_api.h>
+#include <stdint.h>
+
+#include <vector>
+
+#include "ctx.h"
+#include "kernels.h"
+#include "slab_pool.h"
+
+namespace amem {
+
+struct Options {
+  int64_t zero_elide = 1;
+  int64_t verify = 0;
+  int64_t pause_path = 2;                 // 0 direct, 1 staged, 2 auto
+  int64_t dma_min_bytes = 16ll << 20;     // direct path: runs this long go by hipMemcpyAsync
+  int64_t staging_bytes = 256ll << 20;    // each of two device staging buffers
+  int64_t slab_bytes = 256ll << 20;
+  int64_t link_wgs = 96;                  // workgroups of a kernel touching host memory
+  int64_t hbm_wgs = 8192;                 // workgroup cap of device-only kernels
+  int64_t resume_batch_bytes = 64ll << 20;
+  int64_t peer_timeout_ms = 60000;
+};
+Options& options();
+
+// Growable device / pinned-host scratch.
+struct DevBuf {
+  void* p = nullptr;
+  size_t cap = 0;
+  hipError_t ensure(size_t bytes);
+  void release();
+};
+struct PinBuf {
+  void* p = nullptr;
+  size_t cap = 0;
+  hipError_t ensure(size_t bytes);
+  void release();
+};
+
+struct ParkedRegion {
+  uint64_t va;
+  uint64_t size;
+  uint64_t first_chunk;
+  uint64_t nchunks;
+  uint64_t parked_off;    // logical pool offset of the first parked byte
+  uint64_t parked_bytes;
+  uint32_t desc_begin, desc_end;  // range in gather_descs_
+};
+
+class Engine {
+ public:
+  explicit Engine(int dev);
+  ~Engine();
+  hipError_t init();
+
+  // Both are called with Ctx::structure held.
+  int pause(Ctx& c);
+  int resume(Ctx& c);
+  // A region was deleted while paused: drop its parked bytes.
+  void forget(uint64_t va);
+
+  amem_cycle_stats stats() const { return stats_; }
+  uint64_t trim_pool();
+
+  // Standalone kernel entry points (synchronous).
+  hipError_t zero_scan(const amem_extent* ext, uint64_t n, uint8_t* flags, amem_chunk_sum* sums,
+                       float* ms);
+  hipError_t move(bool scatter, const amem_copy_desc* descs, uint64_t n, void* staging,
+                  uint64_t staging_bytes, bool host_side, float* ms);
+  hipError_t probe_link(uint64_t bytes, int reps, double* d2h, double* h2d);
+  hipError_t calib_copy(uint64_t bytes, int reps, float* ms);
+
+ private:
+  hipError_t run_scan(const std::vector<ScanSeg>& segs, uint64_t* nchunks_out, bool want_sums,
+                      float* ms);
+  hipError_t upload_descs(const CopyDesc* descs, size_t n, uint64_t* ntiles_out);
+  hipError_t upload_slab_table();
+  hipError_t pause_copy_direct(Ctx& c, std::vector<Region*>& regs);
+  hipError_t pause_copy_staged(Ctx& c, std::vector<Region*>& regs, bool* used);
+  hipError_t release_local(Ctx& c, Region* r, uint64_t va);
+  hipEvent_t event_at(size_t i);
+
+  int dev_;
+  bool inited_ = false;
+  hipStream_t kstream_ = nullptr;  // kernels
+  hipStream_t dstream_ = nullptr;  // hipMemcpyAsync
+  SlabPool* pool_ = nullptr;
+  size_t slab_table_count_ = 0;
+
+  DevBuf d_segs_, d_prefix_, d_flags_, d_sums_, d_descs_, d_tiles_, d_slabtab_;
+  DevBuf d_staging_[2];
+  PinBuf h_segs_, h_prefix_, h_flags_, h_sums_, h_descs_, h_tiles_, h_slabtab_, h_sums_verify_;
+  std::vector<hipEvent_t> events_;
+
+  // state carried from pause to resume
+  std::vector<ParkedRegion> parked_;
+  std::vector<CopyDesc> gather_descs_;
+  std::vector<ScanSeg> segs_;
+  uint64_t nchunks_ = 0;
+  uint64_t parked_total_ = 0;
+  bool have_sums_ = false;
+
+  amem_cycle_stats stats_ = {};
+};
+
+// Engine of a device, created on first use. Returns nullptr (after an ERROR log) when no
+// GPU is present: there is no host fallback for the data path.
+Engine* engine_for(int dev);
+void destroy_engines();
+
+}  // namespace amem
+#endif

@@ -1,0 +1,328 @@
+#include "ipc.h"
+
+#include <errno.h>
+#include <fcntl.h>
+#include <poll.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <sys/file.h>
+#include <sys/socket.h>
+#include <sys/stat.h>
+#include <sys/un.h>
+#include <unistd.h>
+
+#include <atomic>
+#include <mutex>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include <hip/hip_runtime_api.h>
+
+#include "../../include/amem_nccl.h"
+#include "ctx.h"
+#include "engine.h"
+#include "log.h"
+
+namespace amem {
+
+int amem_groupID_value() { return ::amem_groupID; }
+
+namespace {
+
+// Same numbering as the reference's gmm_ipc_op (gmm_common.h:106-150).
+enum WireOp : int32_t { OP_REGISTER_PEER_INFO = 16, OP_UPDATE_PEER_INFO = 17, OP_RELEASE_PEER_HANDLE = 18 };
+
+struct WireReq {
+  uint32_t magic;
+  int32_t op;
+  int32_t sender_slot;
+  int32_t pid;
+  uint64_t src;  // REGISTER: owner's handle
+  uint64_t tgt;  // REGISTER: importer's VA; UPDATE/RELEASE: receiver's VA
+};
+static constexpr uint32_t kMagic = 0x414d454d;  // "AMEM"
+
+struct Service {
+  std::mutex mtx;  // guards everything below except `stop`
+  int slot = -1;
+  int dev = 0;
+  int lock_fd = -1;
+  int listen_fd = -1;
+  int wake[2] = {-1, -1};
+  std::string sock_path, lock_path;
+  std::thread thr;
+  std::atomic<bool> stop{false};
+  int conn[AMEM_MAX_DEVS];
+  std::mutex conn_mtx[AMEM_MAX_DEVS];
+  Service() { for (int& c : conn) c = -1; }
+};
+// Never destroyed: the service thread may outlive static destruction at exit.
+Service& g_svc = *new Service();
+
+std::string ipc_dir() {
+  const char* d = getenv("GMM_IPC_DIR");  // gmm_server_impl.cpp:78-79
+  return d ? d : "/tmp";
+}
+std::string sock_name(int slot) {
+  char b[256];
+  snprintf(b, sizeof(b), "%s/amem_worker_%x_%d.sock", ipc_dir().c_str(), amem_groupID_value(), slot);
+  return b;
+}
+std::string lock_name(int slot) {
+  char b[256];
+  snprintf(b, sizeof(b), "%s/amem_slot_%x_%d.lock", ipc_dir().c_str(), amem_groupID_value(), slot);
+  return b;
+}
+
+// One message with an optional descriptor; >0 bytes sent, else error.
+ssize_t send_msg(int sock, const void* buf, size_t bytes, int fd) {
+  struct iovec iov = {(void*)buf, bytes};
+  struct msghdr msg = {};
+  union { struct cmsghdr cm; char control[CMSG_SPACE(sizeof(int))]; } cu;
+  msg.msg_iov = &iov;
+  msg.msg_iovlen = 1;
+  if (fd >= 0) {
+    memset(&cu, 0, sizeof(cu));
+    msg.msg_control = cu.control;
+    msg.msg_controllen = sizeof(cu.control);
+    struct cmsghdr* cm = CMSG_FIRSTHDR(&msg);
+    cm->cmsg_level = SOL_SOCKET;
+    cm->cmsg_type = SCM_RIGHTS;
+    cm->cmsg_len = CMSG_LEN(sizeof(int));
+    memcpy(CMSG_DATA(cm), &fd, sizeof(int));
+  }
+  ssize_t r;
+  do { r = sendmsg(sock, &msg, MSG_NOSIGNAL); } while (r < 0 && errno == EINTR);
+  if (r < 0) LOGGER(ERROR, "pid:%d sendmsg failed on connect:%d error:%s", getpid(), sock, strerror(errno));
+  return r;
+}
+
+// Receive exactly `bytes`; a descriptor that rides along is stored in *fd (else -1).
+ssize_t recv_msg(int sock, void* buf, size_t bytes, int* fd) {
+  if (fd) *fd = -1;
+  size_t got = 0;
+  while (got < bytes) {
+    struct iovec iov = {(char*)buf + got, bytes - got};
+    struct msghdr msg = {};
+    union { struct cmsghdr cm; char control[CMSG_SPACE(sizeof(int))]; } cu;
+    msg.msg_iov = &iov;
+    msg.msg_iovlen = 1;
+    msg.msg_control = cu.control;
+    msg.msg_controllen = sizeof(cu.control);
+    ssize_t r = recvmsg(sock, &msg, 0);
+    if (r < 0 && errno == EINTR) continue;
+    if (r <= 0) return r;
+    for (struct cmsghdr* cm = CMSG_FIRSTHDR(&msg); cm; cm = CMSG_NXTHDR(&msg, cm)) {
+      if (cm->cmsg_level == SOL_SOCKET && cm->cmsg_type == SCM_RIGHTS && cm->cmsg_len == CMSG_LEN(sizeof(int))) {
+        int f;
+        memcpy(&f, CMSG_DATA(cm), sizeof(int));
+        if (fd && *fd < 0) *fd = f; else close(f);
+      }
+    }
+    got += (size_t)r;
+  }
+  return (ssize_t)got;
+}
+
+int handle_request(const WireReq& req, int fd) {
+  switch (req.op) {
+    case OP_REGISTER_PEER_INFO:  // gmm_worker_impl.cpp:375-382
+      if (fd >= 0) close(fd);
+      return amem_register_peer_info(req.src, req.tgt, req.sender_slot);
+    case OP_UPDATE_PEER_INFO:    // gmm_worker_impl.cpp:384-390
+      if (fd < 0) {
+        LOGGER(ERROR, "pid:%d recvmsg done but unexpected control header setting", getpid());
+        return 1;
+      }
+      return amem_update_peer_info(req.tgt, fd);
+    case OP_RELEASE_PEER_HANDLE: // gmm_worker_impl.cpp:392-397
+      if (fd >= 0) close(fd);
+      return amem_release_peer_mapping(req.tgt);
+    default:
+      if (fd >= 0) close(fd);
+      LOGGER(ERROR, "worker:%d invalid op:%d", g_svc.slot, req.op);
+      return 1;
+  }
+}
+
+void serve() {
+  if (gpu_present()) (void)hipSetDevice(g_svc.dev);
+  std::vector<struct pollfd> fds;
+  fds.push_back({g_svc.listen_fd, POLLIN, 0});
+  fds.push_back({g_svc.wake[0], POLLIN, 0});
+  while (!g_svc.stop.load()) {
+    int n = poll(fds.data(), fds.size(), -1);
+    if (n < 0) { if (errno == EINTR) continue; break; }
+    if (fds[1].revents) break;
+    if (fds[0].revents & POLLIN) {
+      int c = accept(g_svc.listen_fd, nullptr, nullptr);
+      if (c >= 0) fds.push_back({c, POLLIN, 0});
+    }
+    for (size_t i = 2; i < fds.size();) {
+      if (!(fds[i].revents & (POLLIN | POLLHUP | POLLERR))) { ++i; continue; }
+      WireReq req;
+      int fd = -1;
+      ssize_t r = recv_msg(fds[i].fd, &req, sizeof(req), &fd);
+      if (r != (ssize_t)sizeof(req) || req.magic != kMagic) {
+        // peer went away (gmm_worker_impl.cpp:409-419): drop the connection
+        if (fd >= 0) close(fd);
+        close(fds[i].fd);
+        fds.erase(fds.begin() + i);
+        continue;
+      }
+      int32_t ret = handle_request(req, fd);
+      send_msg(fds[i].fd, &ret, sizeof(ret), -1);
+      ++i;
+    }
+  }
+  for (size_t i = 2; i < fds.size(); ++i) close(fds[i].fd);
+}
+
+bool claim(int slot) {
+  std::string lp = lock_name(slot);
+  int fd = open(lp.c_str(), O_CREAT | O_RDWR | O_CLOEXEC, 0666);
+  if (fd < 0) return false;
+  if (flock(fd, LOCK_EX | LOCK_NB) != 0) { close(fd); return false; }
+  g_svc.lock_fd = fd;
+  g_svc.lock_path = lp;
+  g_svc.slot = slot;
+  return true;
+}
+
+// Connect to the service of `slot`, waiting for it to appear (connect_if_not,
+// gmm_client_impl.cpp:288-347, with a bounded wait instead of an abort).
+int connect_if_not(int slot) {
+  if (g_svc.conn[slot] >= 0) return g_svc.conn[slot];
+  int64_t budget_ms = options().peer_timeout_ms > 0 ? options().peer_timeout_ms : 30000;
+  std::string path = sock_name(slot);
+  struct sockaddr_un addr = {};
+  addr.sun_family = AF_UNIX;
+  strncpy(addr.sun_path, path.c_str(), sizeof(addr.sun_path) - 1);
+  for (int64_t waited = 0;; waited += 20) {
+    int s = socket(AF_UNIX, SOCK_STREAM | SOCK_CLOEXEC, 0);
+    if (s < 0) return -1;
+    if (connect(s, (struct sockaddr*)&addr, sizeof(addr)) == 0) {
+      if (options().peer_timeout_ms > 0) {
+        struct timeval tv = {(time_t)(options().peer_timeout_ms / 1000), (suseconds_t)((options().peer_timeout_ms % 1000) * 1000)};
+        setsockopt(s, SOL_SOCKET, SO_RCVTIMEO, &tv, sizeof(tv));
+        setsockopt(s, SOL_SOCKET, SO_SNDTIMEO, &tv, sizeof(tv));
+      }
+      g_svc.conn[slot] = s;
+      return s;
+    }
+    close(s);
+    if (waited >= budget_ms) break;
+    usleep(20000);
+  }
+  LOGGER(ERROR, "groupID:%d pid:%d error on connecting to %s after retry, error:%s", amem_groupID_value(),
+         getpid(), path.c_str(), strerror(errno));
+  return -1;
+}
+
+int rpc(int slot, const WireReq& req, int fd) {
+  if (slot < 0 || slot >= AMEM_MAX_DEVS) return 1;
+  std::lock_guard<std::mutex> lk(g_svc.conn_mtx[slot]);
+  int s = connect_if_not(slot);
+  if (s < 0) return 1;
+  int32_t ret = 1;
+  if (send_msg(s, &req, sizeof(req), fd) > 0) {
+    if (recv_msg(s, &ret, sizeof(ret), nullptr) != (ssize_t)sizeof(ret)) ret = 1;
+  }
+  if (ret != 0) {
+    // a broken connection is not reused
+    if (errno == EPIPE || errno == ECONNRESET || errno == EAGAIN) { close(s); g_svc.conn[slot] = -1; }
+  }
+  return ret;
+}
+
+}  // namespace
+
+int ipc_slot() { return g_svc.slot; }
+
+int ipc_start(int preferred) {
+  std::lock_guard<std::mutex> lk(g_svc.mtx);
+  if (g_svc.slot >= 0) return g_svc.slot;
+  const char* forced = getenv("AMEM_SLOT");
+  bool ok = false;
+  if (forced) {
+    int s = atoi(forced);
+    ok = s >= 0 && s < AMEM_MAX_DEVS && claim(s);
+  } else {
+    if (preferred < 0 || preferred >= AMEM_MAX_DEVS) preferred = 0;
+    for (int k = 0; k < AMEM_MAX_DEVS && !ok; ++k) ok = claim((preferred + k) % AMEM_MAX_DEVS);
+  }
+  if (!ok) {
+    LOGGER(WARN, "groupID:%d pid:%d no free slot under %s; cross-process regions stay out of pause scope",
+           amem_groupID_value(), getpid(), ipc_dir().c_str());
+    return -1;
+  }
+  g_svc.dev = current_device();
+  g_svc.sock_path = sock_name(g_svc.slot);
+  unlink(g_svc.sock_path.c_str());  // a stale file of a dead holder of this slot
+  g_svc.listen_fd = socket(AF_UNIX, SOCK_STREAM | SOCK_CLOEXEC, 0);
+  struct sockaddr_un addr = {};
+  addr.sun_family = AF_UNIX;
+  strncpy(addr.sun_path, g_svc.sock_path.c_str(), sizeof(addr.sun_path) - 1);
+  if (g_svc.listen_fd < 0 || bind(g_svc.listen_fd, (struct sockaddr*)&addr, sizeof(addr)) != 0 ||
+      listen(g_svc.listen_fd, 64) != 0 || pipe2(g_svc.wake, O_CLOEXEC) != 0) {
+    LOGGER(ERROR, "pid:%d failed to serve on %s error:%s", getpid(), g_svc.sock_path.c_str(), strerror(errno));
+    if (g_svc.listen_fd >= 0) close(g_svc.listen_fd);
+    g_svc.listen_fd = -1;
+    close(g_svc.lock_fd);
+    g_svc.lock_fd = -1;
+    g_svc.slot = -1;
+    return -1;
+  }
+  g_svc.stop.store(false);
+  g_svc.thr = std::thread(serve);
+  LOGGER(DEBUG, "groupID:%d pid:%d serving slot %d on %s", amem_groupID_value(), getpid(), g_svc.slot,
+         g_svc.sock_path.c_str());
+  return g_svc.slot;
+}
+
+void ipc_stop() {
+  std::lock_guard<std::mutex> lk(g_svc.mtx);
+  if (g_svc.slot < 0) return;
+  g_svc.stop.store(true);
+  char b = 1;
+  if (write(g_svc.wake[1], &b, 1) < 0) { /* thread is woken by close below */ }
+  if (g_svc.thr.joinable()) g_svc.thr.join();
+  close(g_svc.listen_fd);
+  close(g_svc.wake[0]);
+  close(g_svc.wake[1]);
+  unlink(g_svc.sock_path.c_str());
+  for (int i = 0; i < AMEM_MAX_DEVS; ++i) {
+    std::lock_guard<std::mutex> lc(g_svc.conn_mtx[i]);
+    if (g_svc.conn[i] >= 0) close(g_svc.conn[i]);
+    g_svc.conn[i] = -1;
+  }
+  unlink(g_svc.lock_path.c_str());
+  close(g_svc.lock_fd);
+  g_svc.lock_fd = g_svc.listen_fd = -1;
+  g_svc.slot = -1;
+}
+
+int peer_register(uint64_t src_handle, uint64_t my_va, int owner_slot) {
+  if (g_svc.slot < 0 || owner_slot == g_svc.slot) return 1;
+  WireReq req = {kMagic, OP_REGISTER_PEER_INFO, g_svc.slot, (int32_t)getpid(), src_handle, my_va};
+  int ret = rpc(owner_slot, req, -1);
+  if (ret != 0)
+    LOGGER(WARN, "groupID:%d pid:%d peer_dev:%d dptr:%llx send|recv error", amem_groupID_value(), getpid(),
+           owner_slot, (unsigned long long)my_va);
+  return ret;
+}
+
+int peer_update(int importer_slot, uint64_t peer_va, int fd) {
+  if (importer_slot == g_svc.slot) return 0;
+  if (g_svc.slot < 0) return 1;
+  WireReq req = {kMagic, OP_UPDATE_PEER_INFO, g_svc.slot, (int32_t)getpid(), 0, peer_va};
+  int ret = rpc(importer_slot, req, fd);
+  if (ret != 0)
+    LOGGER(WARN, "groupID:%d pid:%d peer_dev:%d peer_dptr:%llx newFD:%d send|recv error", amem_groupID_value(),
+           getpid(), importer_slot, (unsigned long long)peer_va, fd);
+  return ret;
+}
+
+}  // namespace amem

@@ -1,0 +1,52 @@
+// Host-visible declarations of the device kernels' argument records and launchers.
+#ifndef AMEM_KERNELS_H_
+#define AMEM_KERNELS_H_
+
+#include <hip/hip_runtime_api.h>
+#include <stdint.h>
+
+namespace amem {
+
+static constexpr uint64_t kChunkBytes = 65536;  // zero-detect / checksum granule
+static constexpr uint64_t kTileBytes = 16384;   // unit of work of the tile mover
+static constexpr uint64_t kDescZero = ~(uint64_t)0;
+
+// One scanned address range; chunk numbering runs range by range.
+struct ScanSeg {
+  uint64_t va;
+  uint64_t bytes;
+};
+
+struct ChunkSum {
+  uint64_t sum64;  // sum of all little-endian uint32 words mod 2^64
+  uint64_t xor64;  // xor of all little-endian uint64 words
+};
+
+// One contiguous copy between a scattered device range and the contiguous side.
+struct CopyDesc {
+  uint64_t va;
+  uint64_t off;    // byte offset on the contiguous side, or kDescZero (scatter: fill zeros)
+  uint64_t bytes;
+};
+
+// The contiguous side: equally sized slabs, slab i covering offsets [i << shift, (i+1) << shift).
+// `base` is an array in device-readable memory.
+struct SlabTable {
+  uint8_t* const* base;
+  uint32_t shift;
+  uint64_t mask;
+};
+
+hipError_t launch_scan(const ScanSeg* d_segs, const uint64_t* d_chunk_prefix, uint32_t nsegs,
+                       uint64_t nchunks, uint8_t* d_flags, ChunkSum* d_sums, uint32_t max_blocks,
+                       hipStream_t stream);
+
+hipError_t launch_move(bool scatter, const CopyDesc* d_descs, const uint64_t* d_tile_prefix,
+                       uint32_t ndescs, uint64_t first_tile, uint64_t ntiles,
+                       const SlabTable& slabs, uint64_t off_base, uint32_t max_blocks,
+                       hipStream_t stream);
+
+hipError_t launch_calib_copy(const void* d_src, void* d_dst, uint64_t bytes, hipStream_t stream);
+
+}  // namespace amem
+#endif

@@ -1,0 +1,227 @@
+// Device kernels of the pause/resume data path, written for gfx950 (CDNA4, wave64).
+//
+// The reference has no device code: its only data movers are cuMemcpyDtoHAsync /
+// cuMemcpyHtoDAsync, one call per region (amem_nccl_plugin/amem_nccl.h:304-327). These
+// kernels exist so that thousands of scattered regions and 64 KiB chunks move at link or
+// HBM rate instead of at per-call rate:
+//
+//   scan_chunks    one wavefront per 64 KiB chunk: is-all-zero flag + (sum64, xor64)
+//   move_tiles     gather-pack / scatter-unpack / zero-fill over a descriptor list
+//   calib_copy     plain copy used to calibrate hardware traffic counters
+//
+// All of it is integer/byte work bound by HBM or by the host link; nothing here is shaped
+// for the matrix cores.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "kernels.h"
+
+namespace amem {
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+static constexpr int kWave = 64;
+static constexpr int kBlock = 256;
+static constexpr int kWavesPerBlock = kBlock / kWave;
+
+// Largest index i in [0, n) with prefix[i] <= x, for a non-decreasing prefix[0..n] with
+// prefix[0] <= x < prefix[n].
+__device__ __forceinline__ uint32_t find_segment(const uint64_t* __restrict__ prefix,
+                                                 uint32_t n, uint64_t x) {
+  uint32_t lo = 0, hi = n;
+  while (hi - lo > 1) {
+    uint32_t mid = (lo + hi) >> 1;
+    if (prefix[mid] <= x) lo = mid; else hi = mid;
+  }
+  return lo;
+}
+
+__device__ __forceinline__ uint64_t wave_reduce_add(uint64_t v) {
+#pragma unroll
+  for (int m = kWave / 2; m >= 1; m >>= 1) {
+    uint32_t lo = __shfl_xor((uint32_t)v, m, kWave);
+    uint32_t hi = __shfl_xor((uint32_t)(v >> 32), m, kWave);
+    v += ((uint64_t)hi << 32) | lo;
+  }
+  return v;
+}
+
+__device__ __forceinline__ uint64_t wave_reduce_xor(uint64_t v) {
+#pragma unroll
+  for (int m = kWave / 2; m >= 1; m >>= 1) {
+    uint32_t lo = __shfl_xor((uint32_t)v, m, kWave);
+    uint32_t hi = __shfl_xor((uint32_t)(v >> 32), m, kWave);
+    v ^= ((uint64_t)hi << 32) | lo;
+  }
+  return v;
+}
+
+__device__ __forceinline__ void accumulate(const u32x4& v, uint64_t& sum, uint64_t& x) {
+  sum += (uint64_t)v.x + (uint64_t)v.y + (uint64_t)v.z + (uint64_t)v.w;
+  x ^= ((uint64_t)v.y << 32 | v.x) ^ ((uint64_t)v.w << 32 | v.z);
+}
+
+// One wavefront per chunk. A full chunk is 64 KiB = 64 lanes x 16 B x 64 rounds; every
+// load instruction of the wave covers 1 KiB of consecutive addresses. Eight loads are
+// issued before the first is consumed so each lane keeps 128 B in flight.
+// A chunk is all-zero exactly when sum64 == 0: the words are unsigned and a chunk holds
+// at most 2^14 of them, so the 64-bit sum cannot wrap.
+__global__ __launch_bounds__(kBlock) void scan_chunks(const ScanSeg* __restrict__ segs,
+                                                      const uint64_t* __restrict__ chunk_prefix,
+                                                      uint32_t nsegs, uint64_t nchunks,
+                                                      uint8_t* __restrict__ flags,
+                                                      ChunkSum* __restrict__ sums) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const uint64_t wave0 = (uint64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x / kWave);
+  const uint64_t nwaves = (uint64_t)gridDim.x * kWavesPerBlock;
+  for (uint64_t c = wave0; c < nchunks; c += nwaves) {
+    const uint32_t s = find_segment(chunk_prefix, nsegs, c);
+    const uint64_t k = c - chunk_prefix[s];
+    const uint64_t seg_bytes = segs[s].bytes;
+    const uint64_t off = k * kChunkBytes;
+    const uint32_t len = (uint32_t)((seg_bytes - off < kChunkBytes) ? (seg_bytes - off) : kChunkBytes);
+    const u32x4* __restrict__ p = (const u32x4*)(segs[s].va + off) + lane;
+    const uint32_t nvec = len >> 4;  // 16-byte vectors in this chunk
+    uint64_t sum = 0, x = 0;
+    uint32_t i = lane;
+    // full rounds of 8 x 1 KiB
+    for (; i + 7 * kWave < nvec; i += 8 * kWave, p += 8 * kWave) {
+      u32x4 v0 = __builtin_nontemporal_load(p);
+      u32x4 v1 = __builtin_nontemporal_load(p + kWave);
+      u32x4 v2 = __builtin_nontemporal_load(p + 2 * kWave);
+      u32x4 v3 = __builtin_nontemporal_load(p + 3 * kWave);
+      u32x4 v4 = __builtin_nontemporal_load(p + 4 * kWave);
+      u32x4 v5 = __builtin_nontemporal_load(p + 5 * kWave);
+      u32x4 v6 = __builtin_nontemporal_load(p + 6 * kWave);
+      u32x4 v7 = __builtin_nontemporal_load(p + 7 * kWave);
+      accumulate(v0, sum, x); accumulate(v1, sum, x);
+      accumulate(v2, sum, x); accumulate(v3, sum, x);
+      accumulate(v4, sum, x); accumulate(v5, sum, x);
+      accumulate(v6, sum, x); accumulate(v7, sum, x);
+    }
+    for (; i < nvec; i += kWave, p += kWave) {
+      u32x4 v = __builtin_nontemporal_load(p);
+      accumulate(v, sum, x);
+    }
+    sum = wave_reduce_add(sum);
+    x = wave_reduce_xor(x);
+    if (lane == 0) {
+      flags[c] = (sum == 0) ? 1 : 0;
+      if (sums) { sums[c].sum64 = sum; sums[c].xor64 = x; }
+    }
+  }
+}
+
+// Resolve a byte offset of the contiguous side to an address. The contiguous side is a
+// list of equally sized slabs (power-of-two bytes); a single buffer is one slab with
+// shift 63.
+__device__ __forceinline__ uint8_t* slab_addr(const SlabTable& t, uint64_t off) {
+  return t.base[off >> t.shift] + (off & t.mask);
+}
+
+// Tile mover. Descriptor d covers tiles [tile_prefix[d], tile_prefix[d+1]) of kTileBytes
+// each (the last tile of a descriptor may be shorter); a launch handles the `ndescs`
+// descriptors whose tiles are [first_tile, first_tile + ntiles). A workgroup takes tiles
+// grid-stride; within a tile, 256 lanes x 16 B = 4 KiB per round, four rounds loaded
+// before any store. `off_base` is subtracted from every descriptor offset, so a sub-range
+// of a long descriptor list can be packed into a buffer that starts at that offset.
+//   MODE 0  gather : staging[off + o] = device[va + o]
+//   MODE 1  scatter: device[va + o] = staging[off + o], or zeros when off == kDescZero
+template <int MODE>
+__global__ __launch_bounds__(kBlock) void move_tiles(const CopyDesc* __restrict__ descs,
+                                                     const uint64_t* __restrict__ tile_prefix,
+                                                     uint32_t ndescs, uint64_t first_tile,
+                                                     uint64_t ntiles, SlabTable slabs,
+                                                     uint64_t off_base) {
+  const uint32_t tid = threadIdx.x;
+  for (uint64_t tt = blockIdx.x; tt < ntiles; tt += gridDim.x) {
+    const uint64_t t = first_tile + tt;
+    const uint32_t d = find_segment(tile_prefix, ndescs, t);
+    const uint64_t o = (t - tile_prefix[d]) * kTileBytes;
+    const uint64_t rem = descs[d].bytes - o;
+    const uint32_t len = (uint32_t)(rem < kTileBytes ? rem : kTileBytes);
+    const uint32_t nvec = len >> 4;
+    const uint64_t off = descs[d].off;
+    u32x4* dev = (u32x4*)(descs[d].va + o);
+    if (MODE == 1 && off == kDescZero) {
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      for (uint32_t i = tid; i < nvec; i += kBlock) __builtin_nontemporal_store(z, dev + i);
+      continue;
+    }
+    u32x4* stg = (u32x4*)slab_addr(slabs, off - off_base + o);
+    const u32x4* __restrict__ src = (MODE == 0) ? dev : stg;
+    u32x4* __restrict__ dst = (MODE == 0) ? stg : dev;
+    uint32_t i = tid;
+    for (; i + 3 * kBlock < nvec; i += 4 * kBlock) {
+      u32x4 a = __builtin_nontemporal_load(src + i);
+      u32x4 b = __builtin_nontemporal_load(src + i + kBlock);
+      u32x4 c = __builtin_nontemporal_load(src + i + 2 * kBlock);
+      u32x4 e = __builtin_nontemporal_load(src + i + 3 * kBlock);
+      __builtin_nontemporal_store(a, dst + i);
+      __builtin_nontemporal_store(b, dst + i + kBlock);
+      __builtin_nontemporal_store(c, dst + i + 2 * kBlock);
+      __builtin_nontemporal_store(e, dst + i + 3 * kBlock);
+    }
+    for (; i < nvec; i += kBlock) {
+      u32x4 a = __builtin_nontemporal_load(src + i);
+      __builtin_nontemporal_store(a, dst + i);
+    }
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void calib_copy(const u32x4* __restrict__ src,
+                                                     u32x4* __restrict__ dst, uint64_t nvec) {
+  uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+  const uint64_t stride = (uint64_t)gridDim.x * kBlock;
+  for (; i < nvec; i += stride) dst[i] = src[i];
+}
+
+// ------------------------------------------------------------------------------------
+// Launchers. Callers have validated: addresses 16-byte aligned, byte counts multiples of
+// 16, prefix arrays consistent with the segment / descriptor arrays, every slab index a
+// descriptor can reach present in the table.
+// ------------------------------------------------------------------------------------
+
+static uint32_t clamp_grid(uint64_t want, uint32_t cap) {
+  if (want < 1) want = 1;
+  return (uint32_t)(want < cap ? want : cap);
+}
+
+hipError_t launch_scan(const ScanSeg* d_segs, const uint64_t* d_chunk_prefix, uint32_t nsegs,
+                       uint64_t nchunks, uint8_t* d_flags, ChunkSum* d_sums, uint32_t max_blocks,
+                       hipStream_t stream) {
+  if (nchunks == 0 || nsegs == 0) return hipSuccess;
+  const uint32_t grid = clamp_grid((nchunks + kWavesPerBlock - 1) / kWavesPerBlock, max_blocks);
+  (void)hipGetLastError();  // an earlier call's sticky error is not this launch's
+  hipLaunchKernelGGL(scan_chunks, dim3(grid), dim3(kBlock), 0, stream, d_segs, d_chunk_prefix,
+                     nsegs, nchunks, d_flags, d_sums);
+  return hipGetLastError();
+}
+
+hipError_t launch_move(bool scatter, const CopyDesc* d_descs, const uint64_t* d_tile_prefix,
+                       uint32_t ndescs, uint64_t first_tile, uint64_t ntiles,
+                       const SlabTable& slabs, uint64_t off_base, uint32_t max_blocks,
+                       hipStream_t stream) {
+  if (ntiles == 0 || ndescs == 0) return hipSuccess;
+  const uint32_t grid = clamp_grid(ntiles, max_blocks);
+  (void)hipGetLastError();
+  if (scatter)
+    hipLaunchKernelGGL(move_tiles<1>, dim3(grid), dim3(kBlock), 0, stream, d_descs, d_tile_prefix,
+                       ndescs, first_tile, ntiles, slabs, off_base);
+  else
+    hipLaunchKernelGGL(move_tiles<0>, dim3(grid), dim3(kBlock), 0, stream, d_descs, d_tile_prefix,
+                       ndescs, first_tile, ntiles, slabs, off_base);
+  return hipGetLastError();
+}
+
+hipError_t launch_calib_copy(const void* d_src, void* d_dst, uint64_t bytes, hipStream_t stream) {
+  const uint64_t nvec = bytes >> 4;
+  if (nvec == 0) return hipSuccess;
+  const uint32_t grid = clamp_grid((nvec + kBlock - 1) / kBlock, 8192);
+  (void)hipGetLastError();
+  hipLaunchKernelGGL(calib_copy, dim3(grid), dim3(kBlock), 0, stream, (const u32x4*)d_src,
+                     (u32x4*)d_dst, nvec);
+  return hipGetLastError();
+}
+
+}  // namespace amem

@@ -1,0 +1,35 @@
+#include "slab_pool.h"
+
+#include "log.h"
+#include "vmm.h"
+
+namespace amem {
+
+SlabPool::SlabPool(uint64_t slab_bytes) {
+  shift_ = 16;
+  while ((1ull << shift_) < slab_bytes && shift_ < 40) ++shift_;
+  slab_bytes_ = 1ull << shift_;
+}
+
+SlabPool::~SlabPool() { trim(); }
+
+hipError_t SlabPool::ensure(uint64_t bytes) {
+  while (capacity() < bytes) {
+    void* p = nullptr;
+    hipError_t e = CHECK_HIP(hipHostMalloc(&p, slab_bytes_, hipHostMallocDefault));
+    if (e != hipSuccess) return e;
+    slabs_.push_back((uint8_t*)p);
+    LOGGER(DEBUG, "slab pool: +1 slab of %llu MiB, %zu slabs", (unsigned long long)(slab_bytes_ >> 20),
+           slabs_.size());
+  }
+  return hipSuccess;
+}
+
+uint64_t SlabPool::trim() {
+  uint64_t freed = capacity();
+  for (uint8_t* p : slabs_) (void)CHECK_HIP(hipHostFree(p));
+  slabs_.clear();
+  return freed;
+}
+
+}  // namespace amem

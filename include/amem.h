@@ -1,0 +1,347 @@
+/*
+ * amem.h — C ABI of the MI355X AMem pause/resume engine (libamem_nccl.so.1).
+ *
+ * Plain C: fixed-width integers, pointers and sizes only. Device virtual addresses and
+ * physical-allocation handles cross this boundary as opaque uint64_t (the reference's
+ * CUdeviceptr / CUmemGenericAllocationHandle are both `unsigned long long`); inside the
+ * library they are cast to hipDeviceptr_t / hipMemGenericAllocationHandle_t.
+ *
+ * Every entry point that replaces a function of the reference cites it as
+ * `amem_nccl_plugin/<file>:<line>`. The same library also exports the reference's
+ * C++-linkage names with identical signatures (see amem_nccl.h) so that code compiled
+ * against the reference header links unchanged.
+ *
+ * Error convention (reference: gmm_cuda_common.h:38-55, amem_nccl.cpp return paths):
+ * int 0 = success, non-zero = failure or rejection. While the engine is disabled
+ * (AMEM_ENABLE unset or 0, or NCCL_CUMEM_ENABLE=0; amem_nccl.cpp:711-718) every
+ * reference-mirroring entry point returns 0 and does nothing.
+ */
+#ifndef AMEM_H_
+#define AMEM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+/* The library is built with hidden visibility; everything declared here is exported. */
+#pragma GCC visibility push(default)
+
+#define AMEM_MAX_DEVS 8    /* amem_nccl.h:32; also the length of peers[] */
+#define AMEM_MAX_CALLER 16 /* amem_nccl.h:33 */
+#define AMEM_CHUNK_BYTES 65536u /* zero-detect / checksum chunk */
+
+/* amem_nccl.h:39-49 */
+enum amem_alloc_state {
+  AMEM_STATE_INVALID = 0,
+  AMEM_STATE_ALLOC = 1,
+  AMEM_STATE_OFFLOADING = 2,
+  AMEM_STATE_HOLE = 3,
+  AMEM_STATE_PRELOADING = 4,
+  AMEM_STATE_REMAPPED = 5,
+  AMEM_STATE_MAX = 6
+};
+
+/* amem_nccl.h:52-64. type <= LOCAL_SYMM means the region owns its bytes. */
+enum amem_alloc_type {
+  AMEM_TYPE_LOCAL = 0,
+  AMEM_TYPE_LOCAL_POSIX = 0,
+  AMEM_TYPE_LOCAL_FABRIC = 1,
+  AMEM_TYPE_LOCAL_SYMM = 2,
+  AMEM_TYPE_PEER_POSIX = 3,
+  AMEM_TYPE_PEER_FABRIC = 4,
+  AMEM_TYPE_PEER_SYMM = 5,
+  AMEM_TYPE_MAX = 6
+};
+
+/* amem_nccl.h:67-80 */
+enum amem_caller {
+  AMEM_CALLER_DEFAULT = 0,
+  AMEM_CALLER_P2P = 1,
+  AMEM_CALLER_FABRIC = 2,
+  AMEM_CALLER_POSIX = 3,
+  AMEM_CALLER_SYMM = 4,
+  AMEM_CALLER_NVLS = 5,
+  AMEM_CALLER_RESERVED = 6,
+  AMEM_CALLER_P2P_PEER = 7,
+  AMEM_CALLER_RESERVED2 = 8,
+  AMEM_CALLER_PROXY = 9,
+  AMEM_CALLER_SYMM_PEER = 10,
+  AMEM_CALLER_MAX = AMEM_MAX_CALLER
+};
+
+/* ---------------------------------------------------------------------------------------
+ * 1. The allocator hook and the per-process region registry
+ * ------------------------------------------------------------------------------------- */
+
+/* Record one VMM allocation (local) or one imported mapping (peer).
+ * Replaces amem_addAllocInfo, amem_nccl.cpp:102-269 (declared amem_nccl.h:344-346).
+ * Returns 0; 1 when called while paused (:133-137) or when a peer mapping's owner cannot
+ * be determined (:245-256); the RPC status when registering with the owner fails, in which
+ * case the entry is erased again (:209-220).
+ * For peer types `peer_dev` names the owner: the owner's slot (see amem_get_slot) when
+ * several processes share one GPU, which is the only multi-process layout this library
+ * runs; -1 asks the library to detect it from the handle. */
+int amem_add_alloc_info(uint64_t va, uint64_t size, int type, int dev, uint64_t handle,
+                        int peer_dev, uint64_t peer_handle, void* user_info, int caller);
+
+/* Forget a region before its VA is freed. Replaces amem_delAllocInfo,
+ * amem_nccl.cpp:414-448. handle == 0 asks the library to look the handle up from the
+ * mapping. Always returns 0. The per-caller byte counter that the add incremented is the
+ * one decremented (the reference indexes by this call's `caller` argument instead, which
+ * its hooks hard-code to 0; the argument is accepted and ignored here). */
+int amem_del_alloc_info(uint64_t va, uint64_t handle, int caller);
+
+/* Add `n` extra physical-handle references that pause must also drop.
+ * Replaces amem_addRefcount, amem_nccl.cpp:332-356. 0 ok, 1 region not found. */
+int amem_add_refcount(void* va, int n);
+
+/* Same-process peer record: peers[peer_dev] = peer_va, hasPeer = true.
+ * Replaces amem_addPeerInfo, amem_nccl.cpp:359-381. 0 ok, 1 not found. */
+int amem_add_peer_info(uint64_t src_va, uint64_t peer_va, int peer_dev);
+
+/* Owner-side half of an import: find the local region that `src_handle` backs and
+ * record the importer's VA. Replaces amem_registerPeerInfo, amem_nccl.cpp:297-329.
+ * Runs on the IPC service thread when an importer registers. 0 ok, 1 not found. */
+int amem_register_peer_info(uint64_t src_handle, uint64_t peer_va, int peer_dev);
+
+/* Importer-side half of a resume: import `shared_fd`, map it at the region's original VA,
+ * close the fd. Replaces amem_updatePeerInfo, amem_nccl.cpp:385-409. 0 ok. */
+int amem_update_peer_info(uint64_t va, int shared_fd);
+
+/* Paused gate. Replaces amem_checkPaused, amem_nccl.cpp:452-464. Returns 1 when paused. */
+int amem_check_paused(int warn);
+
+/* Group id, settable only before the first tracked allocation.
+ * Replace amem_setGroupID / amem_getGroupID, amem_nccl.cpp:679-703. set: 0 ok, 1 too late. */
+int amem_set_group_id(int id);
+void amem_get_group_id(int* id);
+
+/* Per-caller byte statistics to stdout. Replaces amem_dumpAllocStats, amem_nccl.cpp:82-99. */
+void amem_dump_alloc_stats(int verbose);
+
+/* ---------------------------------------------------------------------------------------
+ * 2. Pause / resume
+ * ------------------------------------------------------------------------------------- */
+
+/* Park the bytes of every local region of the current device in pinned host memory,
+ * then unmap and release all physical memory behind every tracked VA (imported mappings
+ * first). VAs stay reserved. Replaces amem_memPause, amem_nccl.cpp:467-574.
+ * Idempotent; returns 0, or non-zero when a HIP call failed (the reference always
+ * returns 0 and only prints driver errors). */
+int amem_mem_pause(int pid, uint64_t tag);
+
+/* Re-create physical memory at the identical VAs, restore the bytes, re-export to every
+ * recorded importer and wait until every mapping this process imports is back.
+ * Replaces amem_memResume, amem_nccl.cpp:577-677. Idempotent. */
+int amem_mem_resume(int pid, uint64_t tag);
+
+/* The five public names the patched NCCL exports (nccl_patch/nccl_2.27.5-1.diff:68-112,
+ * :337-351). `comm` is ignored. ncclPause/ncclResume report 0 whatever the inner call
+ * returned, as the reference does (:70-88); ncclSetGroupID returns the inner int (:102-105). */
+int ncclPause(void* comm);
+int ncclResume(void* comm);
+int ncclMemStats(void);
+int ncclSetGroupID(int id);
+int ncclGetGroupID(int* id);
+
+/* ---------------------------------------------------------------------------------------
+ * 3. VMM allocation helpers
+ * ------------------------------------------------------------------------------------- */
+
+/* Reserve a VA range, create device memory exportable as a POSIX fd, map it and grant
+ * read/write to `dev`; unwinds on failure. `bytes` is rounded up to 2 MiB.
+ * Replaces gmm_cuda_vmm_alloc, gmm_cuda_mem_impl.cpp:237-273 (call order and unwind of
+ * gpu_vmm_alloc, :84-194). Does not register the region. */
+int amem_vmm_alloc(uint64_t bytes, int dev, uint64_t* va, uint64_t* handle,
+                   uint64_t* alloc_size);
+
+/* Unmap, release and free the VA range. Works for a region in any state: a region the
+ * engine has paused (no physical memory) only has its reservation freed.
+ * Replaces gmm_cuda_vmm_free / gpu_vmm_free, gmm_cuda_mem_impl.cpp:196-222, :275-283.
+ * `handle` may be 0: the current handle is then looked up from the mapping, which is what
+ * a caller must do after a resume replaced the handle it created. */
+int amem_vmm_free(uint64_t va, uint64_t alloc_size, uint64_t handle);
+
+/* Export a handle as a POSIX fd / import one and map it at a fresh VA.
+ * Counterparts of the export in amem_cuAllocAndExport (amem_nccl.h:186-190) and of
+ * amem_importAndMap (amem_nccl.h:216-234) for the initial, caller-side exchange that the
+ * reference leaves to NCCL. amem_vmm_import does not close `fd`. */
+int amem_vmm_export(uint64_t handle, int* fd);
+int amem_vmm_import(int fd, uint64_t size, int dev, uint64_t* va, uint64_t* handle);
+
+/* ---------------------------------------------------------------------------------------
+ * 4. Registry inspection (the reference exposes these as public data members of
+ *    gmm_client_ctx, gmm_client.h:136-152, and fields of amem_allocMdata, amem_nccl.h:87-138)
+ * ------------------------------------------------------------------------------------- */
+
+typedef struct amem_region_info {
+  uint64_t va;
+  uint64_t handle;
+  uint64_t mc_handle;
+  uint64_t alloc_sz;
+  uint64_t tags;
+  uint64_t peers[AMEM_MAX_DEVS];
+  uint64_t cpu_addr;     /* host address of the first parked byte; 0 before the first pause */
+  uint64_t user_info;
+  uint64_t parked_bytes; /* bytes of this region held in host memory by the last pause */
+  uint64_t handle_gen;   /* number of physical handles this VA has had (1 after add) */
+  int32_t dev;
+  int32_t pid;
+  int32_t refcount;
+  int32_t shared_fd;
+  int32_t type;
+  int32_t state;
+  int32_t has_peer;
+  int32_t oos_flag;
+} amem_region_info;
+
+typedef struct amem_counters {
+  int64_t release_local_cnt;
+  int64_t release_shadow_cnt;
+  int64_t offload_cnt;
+  int64_t smoke_log;
+  uint64_t alloc_bytes[AMEM_MAX_CALLER];
+  uint64_t del_bytes;
+  uint64_t pause_cnt;
+  uint64_t resume_cnt;
+  int32_t paused;
+  int32_t group_id;
+  int32_t enabled;
+  int32_t slot;
+} amem_counters;
+
+/* Number of regions tracked for `dev`; entries are ordered by ascending VA. */
+int64_t amem_region_count(int dev);
+/* Copy the `index`-th region (ascending VA) of `dev`. 0 ok, 1 out of range. */
+int amem_region_at(int dev, int64_t index, amem_region_info* out);
+/* Copy the region whose key is `va`. 0 ok, 1 not found. */
+int amem_region_find(int dev, uint64_t va, amem_region_info* out);
+/* handleTable lookup: VA that `handle` backs (local regions only), 0 if absent. */
+uint64_t amem_handle_lookup(int dev, uint64_t handle);
+int64_t amem_handle_count(int dev);
+void amem_get_counters(amem_counters* out);
+
+/* Per-phase timing of the most recent pause and resume, in milliseconds unless named. */
+typedef struct amem_cycle_stats {
+  double pause_ms, resume_ms;
+  double pause_scan_ms;     /* K1 launch -> flags on host */
+  double pause_plan_ms;     /* host: runs, staging layout, descriptor upload */
+  double pause_copy_ms;     /* first copy enqueued -> last byte in host memory */
+  double pause_unmap_ms;    /* host time inside hipMemUnmap + hipMemRelease */
+  double resume_map_ms;     /* host time inside hipMemCreate + hipMemMap + hipMemSetAccess */
+  double resume_copy_ms;    /* first copy enqueued -> last byte in device memory */
+  double resume_peer_ms;    /* export + notify importers + wait for owners */
+  double k1_ms;             /* device time of the zero/checksum scan (HIP events) */
+  double k2_ms;             /* device time of gather-pack launches (sum) */
+  double k3_ms;             /* device time of scatter-unpack launches (sum) */
+  uint64_t k1_launches, k2_launches, k3_launches;
+  uint64_t footprint_bytes; /* sum of allocSz over local regions */
+  uint64_t parked_bytes;    /* bytes that crossed the host link per leg */
+  uint64_t zero_chunks, total_chunks;
+  uint64_t local_regions, peer_regions;
+  uint64_t dma_bytes;       /* of parked_bytes, how much moved by hipMemcpyAsync */
+  uint64_t kernel_bytes;    /* of parked_bytes, how much moved by the pack/unpack kernels */
+  uint64_t slab_bytes;      /* pinned host memory held by the pool */
+  uint64_t verify_mismatch; /* chunks whose checksum differed after resume (verify mode) */
+} amem_cycle_stats;
+void amem_get_cycle_stats(amem_cycle_stats* out);
+
+/* ---------------------------------------------------------------------------------------
+ * 5. Engine controls without a reference counterpart
+ * ------------------------------------------------------------------------------------- */
+
+/* Turn the engine on or off at run time (the reference reads AMEM_ENABLE once at load,
+ * amem_nccl.cpp:711). Only allowed while nothing is tracked. 0 ok, 1 rejected. */
+int amem_set_enabled(int on);
+
+/* Tunables. Unknown name or bad value returns 1. Names:
+ *   "zero_elide"      0/1   skip all-zero 64 KiB chunks (default 1)
+ *   "verify"          0/1   re-scan after resume and compare checksums (default 0)
+ *   "pause_path"      0 = pack kernel writes pinned host memory directly,
+ *                     1 = pack into device staging, then large hipMemcpyAsync, unmap overlapped
+ *                     2 = choose 1 when staging memory can be allocated, else 0 (default)
+ *   "dma_min_bytes"   extents at least this long use hipMemcpyAsync in the direct path
+ *   "staging_bytes"   size of each of the two device staging buffers
+ *   "slab_bytes"      size of one pinned host slab (power of two)
+ *   "link_wgs"        workgroups of a kernel that reads or writes host memory
+ *   "peer_timeout_ms" how long resume waits for owners before failing (0 = forever) */
+int amem_set_option(const char* name, int64_t value);
+int64_t amem_get_option(const char* name);
+
+/* Release the pinned host pool (only while not paused). Returns bytes freed. */
+uint64_t amem_pool_trim(void);
+
+/* Tear the per-process context down to the state before the first tracked allocation:
+ * registry emptied (nothing is unmapped or freed), pool released, IPC service stopped,
+ * counters zeroed. Rejected (1) while paused. The reference has only x_fini (:726-729). */
+int amem_shutdown(void);
+
+/* Slot of this process within its group on this node: index into peers[] that importers
+ * pass as `peer_dev`. Taken from AMEM_SLOT or claimed first-free when the IPC service
+ * starts. Returns -1 before that. amem_ipc_start starts the service explicitly (it is
+ * otherwise started by the first add of a peer-type region or by amem_get_slot). */
+int amem_ipc_start(void);
+int amem_get_slot(void);
+
+/* ---------------------------------------------------------------------------------------
+ * 6. The device kernels, callable on their own (no reference counterpart: the reference
+ *    moves bytes only with cuMemcpyDtoHAsync / cuMemcpyHtoDAsync, amem_nccl.h:304-327)
+ * ------------------------------------------------------------------------------------- */
+
+typedef struct amem_extent {
+  uint64_t va;    /* device address, 16-byte aligned */
+  uint64_t bytes; /* multiple of 16 */
+} amem_extent;
+
+typedef struct amem_chunk_sum {
+  uint64_t sum64; /* sum of all little-endian uint32 words, mod 2^64 */
+  uint64_t xor64; /* xor of all little-endian uint64 words */
+} amem_chunk_sum;
+
+/* Zero-chunk detector + checksum. Every extent is cut into 64 KiB chunks (the last one
+ * of an extent may be shorter); chunks are numbered extent by extent. Writes one flag
+ * byte (1 = all bytes zero) and one checksum pair per chunk to host arrays of
+ * amem_chunk_count(extents, n) entries. `sums` may be NULL. Returns 0, or a HIP error. */
+uint64_t amem_chunk_count(const amem_extent* extents, uint64_t n);
+int amem_zero_scan(const amem_extent* extents, uint64_t n, uint8_t* flags,
+                   amem_chunk_sum* sums, float* kernel_ms);
+
+typedef struct amem_copy_desc {
+  uint64_t va;      /* scattered side: device address, 16-byte aligned */
+  uint64_t off;     /* contiguous side: byte offset into the staging buffer, 16-byte aligned;
+                       AMEM_DESC_ZERO on unpack means "write zeros to va" */
+  uint64_t bytes;   /* multiple of 16 */
+} amem_copy_desc;
+#define AMEM_DESC_ZERO (~(uint64_t)0)
+
+/* Gather-pack: staging[off .. off+bytes) = device[va .. va+bytes) for every descriptor.
+ * Scatter-unpack: the reverse, plus zero fill for AMEM_DESC_ZERO descriptors.
+ * `staging` is a device pointer or a hipHostMalloc pointer; `host_side` non-zero selects
+ * the launch shape tuned for the host link. Descriptor arrays are host memory.
+ * Synchronous. Returns 0, or a HIP error. */
+int amem_gather_pack(const amem_copy_desc* descs, uint64_t n, void* staging,
+                     uint64_t staging_bytes, int host_side, float* kernel_ms);
+int amem_scatter_unpack(const amem_copy_desc* descs, uint64_t n, const void* staging,
+                        uint64_t staging_bytes, int host_side, float* kernel_ms);
+
+/* Measured host-link roofline: best-of-`reps` hipMemcpy of `bytes` between device memory
+ * and a pinned host buffer, each direction, in GB/s (1e9 bytes per second). */
+int amem_probe_link(uint64_t bytes, int reps, double* d2h_gbps, double* h2d_gbps);
+
+/* Plain device-to-device copy kernel of `bytes` (multiple of 16), used to calibrate the
+ * FETCH_SIZE / WRITE_SIZE hardware counters against a known traffic. */
+int amem_calib_copy(uint64_t bytes, int reps, float* kernel_ms);
+
+/* Raw byte access for tests and benchmarks (hipMemcpy wrappers, synchronous). */
+int amem_copy_to_device(uint64_t va, const void* host, uint64_t bytes);
+int amem_copy_from_device(void* host, uint64_t va, uint64_t bytes);
+int amem_device_mem_info(uint64_t* free_bytes, uint64_t* total_bytes);
+int amem_device_count(void);
+
+#pragma GCC visibility pop
+#ifdef __cplusplus
+} /* extern "C" */
+#endif
+#endif /* AMEM_H_ */

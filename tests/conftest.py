@@ -1,0 +1,66 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# The library reads these once, when it is loaded (reference: amem_nccl.cpp:711-718).
+os.environ.setdefault("AMEM_ENABLE", "1")
+os.environ.setdefault("GMM_LOG", "1")
+os.environ.setdefault("GMM_IPC_DIR", os.environ.get("TMPDIR", "/tmp"))
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+def _built():
+    from asystem_amem_amd import binding, footprint
+    import oracle
+    return all(os.path.exists(p) for p in (binding.LIB_PATH, footprint.LIB_PATH, oracle.LIB_PATH))
+
+
+@pytest.fixture(scope="session", autouse=True)
+def _libraries():
+    """Tests load what is built; they build only when nothing is."""
+    if not _built():
+        import __graft_entry__
+        __graft_entry__.build()
+
+
+@pytest.fixture(scope="session")
+def lib():
+    from asystem_amem_amd import binding
+    return binding.load()
+
+
+@pytest.fixture(scope="session")
+def orc():
+    import oracle
+    return oracle.load()
+
+
+@pytest.fixture()
+def fresh(lib):
+    """Engine context reset to the state before the first tracked allocation."""
+    assert lib.amem_shutdown() == 0
+    lib.amem_set_enabled(1)
+    yield lib
+    assert lib.amem_shutdown() == 0
+
+
+@pytest.fixture()
+def fresh_orc(orc):
+    orc.oracle_reset()
+    yield orc
+    orc.oracle_reset()
+
+
+@pytest.fixture(scope="session")
+def gpu(lib):
+    if lib.amem_device_count() < 1:
+        pytest.skip("no GPU visible")
+    return lib

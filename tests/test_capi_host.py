@@ -1,0 +1,179 @@
+"""Host-side tests of the shipped library, no GPU needed: it loads, exports every symbol the
+headers declare (and the reference's own mangled names), its registry behaves exactly like
+the oracle's on the same sequence of calls, and the data path refuses to run without a GPU."""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import pytest
+
+import oracle as O
+from asystem_amem_amd import binding as B
+from asystem_amem_amd import harness as H
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+MiB = 1 << 20
+
+
+def exported_symbols():
+    out = subprocess.run(["nm", "-D", "--defined-only", B.LIB_PATH], check=True, capture_output=True, text=True).stdout
+    return {line.split()[-1] for line in out.splitlines() if line.strip()}
+
+
+def declared_c_functions(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return set(re.findall(r"\b((?:amem|nccl)[A-Za-z0-9_]*)\s*\(", text))
+
+
+def test_library_exports_every_declared_symbol(lib):
+    syms = exported_symbols()
+    declared = declared_c_functions("amem.h")
+    assert len(declared) >= 45
+    missing = sorted(d for d in declared if d not in syms)
+    assert not missing, missing
+    assert set(B.c_abi_names()) == declared, set(B.c_abi_names()) ^ declared
+    # the reference's C++-linkage names, exactly as its library exports them
+    for m in B.MANGLED_REFERENCE_SYMBOLS:
+        assert m in syms, m
+    for name in declared_c_functions("amem_nccl.h"):
+        assert any(name in s and s.startswith("_Z") for s in syms), name
+    # nothing internal leaks out
+    leaked = [s for s in syms if s.startswith("_ZN4amem") and "scan_chunks" not in s and "calib_copy" not in s
+              and "move_tiles" not in s]
+    assert not leaked, leaked
+
+
+def test_soname(lib):
+    out = subprocess.run(["readelf", "-d", B.LIB_PATH], check=True, capture_output=True, text=True).stdout
+    assert "libamem_nccl.so.1" in out  # reference: amem_nccl_plugin/Makefile:19
+
+
+def both(fresh, orc):
+    """Run the same registry call on the engine and on the oracle and insist on the same result."""
+    class Pair:
+        def add(self, va, size=2 * MiB, type_=0, handle=None, peer_dev=-1, peer_handle=0, user=0, caller=1, expect=None):
+            h = handle if handle is not None else va + 1
+            a = fresh.amem_add_alloc_info(va, size, type_, 0, h, peer_dev, peer_handle, user or None, caller)
+            b = orc.oracle_add_alloc_info(0, va, size, type_, 0, h, peer_dev, peer_handle, user, caller)
+            assert a == b, ("add", hex(va), a, b)
+            if expect is not None:
+                assert a == expect
+            return a
+
+        def check(self):
+            et, ot = H.region_table(fresh, 0), O.region_table(orc, 0)
+            assert set(et) == set(ot)
+            for va in et:
+                for f in ("handle", "mc_handle", "alloc_sz", "tags", "peers", "user_info", "dev", "pid", "refcount",
+                          "shared_fd", "type", "state", "has_peer", "oos_flag", "cpu_addr"):
+                    assert et[va][f] == ot[va][f], (hex(va), f, et[va][f], ot[va][f])
+            ec, oc = H.counters(fresh), O.counters(orc, 0)
+            for k in ("release_local_cnt", "release_shadow_cnt", "offload_cnt", "smoke_log", "alloc_bytes", "del_bytes",
+                      "pause_cnt", "resume_cnt", "paused", "group_id"):
+                assert ec[k] == oc[k], (k, ec[k], oc[k])
+            assert fresh.amem_handle_count(0) == oc["handle_count"]
+    return Pair()
+
+
+def test_registry_matches_oracle_call_for_call(fresh, fresh_orc):
+    lib, orc = fresh, fresh_orc
+    p = both(lib, orc)
+    assert lib.amem_set_group_id(170) == orc.oracle_set_group_id(0, 170) == 0
+    p.add(0x7f0000000000, 4 * MiB, caller=1, handle=0xA1, user=0x1234, expect=0)
+    p.add(0x7f0010000000, 2 * MiB, caller=3, handle=0xA2, expect=0)
+    p.add(0x7f0020000000, 16 * MiB, type_=2, caller=4, handle=0xA3, peer_handle=0x55, expect=0)   # symmetric: local
+    p.add(0x7f0030000000, 2 * MiB, caller=99, handle=0xA4, expect=0)                               # caller out of range
+    p.check()
+    assert lib.amem_set_group_id(200) == orc.oracle_set_group_id(0, 200) == 1
+    g = C.c_int(-1)
+    lib.amem_get_group_id(C.byref(g))
+    assert g.value == orc.oracle_get_group_id(0) == 170
+    p.add(0x7f0000000000, 8 * MiB, caller=7, handle=0xB1, user=0x99, expect=0)                      # re-registration
+    p.check()
+    for h in (0xA1, 0xB1, 0xA2, 0xDEAD):
+        assert lib.amem_handle_lookup(0, h) == orc.oracle_handle_lookup(0, 0, h)
+    assert lib.amem_add_refcount(C.c_void_p(0x7f0010000000), 3) == orc.oracle_add_refcount(0, 0x7f0010000000, 3) == 0
+    assert lib.amem_add_refcount(C.c_void_p(0x123), 1) == orc.oracle_add_refcount(0, 0x123, 1) == 1
+    assert lib.amem_add_peer_info(0x7f0010000000, 0x5000, 6) == orc.oracle_add_peer_info(0, 0x7f0010000000, 0x5000, 6) == 0
+    assert lib.amem_add_peer_info(0x123, 0x5000, 6) == orc.oracle_add_peer_info(0, 0x123, 0x5000, 6) == 1
+    assert lib.amem_register_peer_info(0xA3, 0x6000, 2) == orc.oracle_register_peer_info(0, 0xA3, 0x6000, 2) == 0
+    assert lib.amem_register_peer_info(0xBAD, 0x6000, 2) == orc.oracle_register_peer_info(0, 0xBAD, 0x6000, 2) == 1
+    p.check()
+    # imported mappings: own slot as owner is refused, unknown owner is dropped
+    slot = lib.amem_get_slot()
+    p.add(0x7f0040000000, 2 * MiB, type_=3, caller=7, handle=0xC1, peer_dev=slot if slot >= 0 else 0, peer_handle=0xA2, expect=1)
+    p.add(0x7f0050000000, 2 * MiB, type_=3, caller=9, handle=0xC2, peer_dev=-1, peer_handle=0xA2, expect=1)
+    p.check()
+    assert lib.amem_del_alloc_info(0x7f0010000000, 0xA2, 0) == orc.oracle_del_alloc_info(0, 0x7f0010000000, 0xA2, 0) == 0
+    assert lib.amem_del_alloc_info(0x7f0030000000, 0xA4, -1) == orc.oracle_del_alloc_info(0, 0x7f0030000000, 0xA4, -1) == 0
+    assert lib.amem_del_alloc_info(0, 0, 0) == orc.oracle_del_alloc_info(0, 0, 0, 0) == 0
+    assert lib.amem_del_alloc_info(0x999000, 0x1, 0) == orc.oracle_del_alloc_info(0, 0x999000, 0x1, 0) == 0
+    p.check()
+    assert lib.amem_check_paused(0) == orc.oracle_check_paused(0) == 0
+
+
+def test_region_order_and_find(fresh):
+    lib = fresh
+    vas = [0x7f0030000000, 0x7f0010000000, 0x7f0020000000]
+    for v in vas:
+        assert lib.amem_add_alloc_info(v, 2 * MiB, 0, 0, v + 1, -1, 0, None, 1) == 0
+    info = B.RegionInfo()
+    got = []
+    for k in range(lib.amem_region_count(0)):
+        assert lib.amem_region_at(0, k, C.byref(info)) == 0
+        got.append(info.va)
+    assert got == sorted(vas)                         # iteration order is defined: ascending VA
+    assert lib.amem_region_at(0, 3, C.byref(info)) == 1
+    assert lib.amem_region_find(0, vas[0], C.byref(info)) == 0 and info.handle == vas[0] + 1 and info.handle_gen == 1
+    assert lib.amem_region_find(0, 0x1, C.byref(info)) == 1
+    assert lib.amem_region_count(5) == 0
+
+
+def test_disabled_engine_ignores_everything(fresh):
+    lib = fresh
+    assert lib.amem_set_enabled(0) == 0
+    assert lib.amem_add_alloc_info(0x7f0000000000, 2 * MiB, 0, 0, 1, -1, 0, None, 1) == 0
+    assert lib.amem_region_count(0) == 0
+    assert lib.amem_mem_pause(0, 0) == 0 and lib.amem_mem_resume(0, 0) == 0 and lib.amem_check_paused(1) == 0
+    assert lib.amem_set_group_id(5) == 0
+    g = C.c_int(-7)
+    lib.amem_get_group_id(C.byref(g))
+    assert g.value == -7                              # amem_getGroupID leaves *id alone when disabled (:698-700)
+    assert lib.ncclPause(None) == 0 and lib.ncclResume(None) == 0 and lib.ncclMemStats() == 0
+    assert lib.amem_set_enabled(1) == 0
+    assert lib.amem_add_alloc_info(0x7f0000000000, 2 * MiB, 0, 0, 1, -1, 0, None, 1) == 0
+    assert lib.amem_set_enabled(0) == 1               # not while something is tracked
+
+
+def test_options(lib):
+    assert lib.amem_set_option(b"no_such_option", 1) == 1
+    assert lib.amem_set_option(b"slab_bytes", 3 << 20) == 1          # not a power of two
+    old = lib.amem_get_option(b"dma_min_bytes")
+    assert lib.amem_set_option(b"dma_min_bytes", 1 << 20) == 0 and lib.amem_get_option(b"dma_min_bytes") == 1 << 20
+    assert lib.amem_set_option(b"dma_min_bytes", old) == 0
+    assert lib.amem_get_option(b"nope") == -1
+
+
+def test_data_path_fails_loudly_without_gpu(fresh):
+    lib = fresh
+    if lib.amem_device_count() > 0:
+        pytest.skip("a GPU is visible")
+    assert lib.amem_add_alloc_info(0x7f0000000000, 2 * MiB, 0, 0, 1, -1, 0, None, 1) == 0
+    assert lib.amem_mem_pause(0, 0) != 0              # no host fallback: an error, and not paused
+    assert lib.amem_check_paused(0) == 0
+    va, h, asz = C.c_uint64(), C.c_uint64(), C.c_uint64()
+    assert lib.amem_vmm_alloc(2 * MiB, 0, C.byref(va), C.byref(h), C.byref(asz)) != 0
+    ext = (B.Extent * 1)(B.Extent(0x1000, 65536))
+    flag = (C.c_uint8 * 1)()
+    assert lib.amem_zero_scan(ext, 1, flag, None, None) != 0
+    d, u = C.c_double(), C.c_double()
+    assert lib.amem_probe_link(1 << 20, 1, C.byref(d), C.byref(u)) != 0
+
+
+def test_missing_library_is_an_error(monkeypatch):
+    monkeypatch.setattr(B, "_lib", None)
+    with pytest.raises(RuntimeError):
+        B.load("/nonexistent/libamem_nccl.so.1")
+    monkeypatch.undo()

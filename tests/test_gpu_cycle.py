@@ -1,0 +1,258 @@
+"""Pause/resume on the GPU through the C ABI: restored bytes identical, identical VAs, region
+table and counters equal to the oracle's after the same calls, physical memory really released,
+every option path, and the edge cases of the reference's state machine."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle as O
+from asystem_amem_amd import binding as B
+from asystem_amem_amd import harness as H
+from asystem_amem_amd.footprint import CHUNK, Footprint
+
+pytestmark = pytest.mark.gpu
+MiB = 1 << 20
+
+
+@pytest.fixture()
+def eng(gpu, fresh):
+    defaults = {k: fresh.amem_get_option(k) for k in (b"zero_elide", b"verify", b"pause_path", b"dma_min_bytes",
+                                                       b"staging_bytes", b"resume_batch_bytes")}
+    yield fresh
+    fresh.amem_mem_resume(0, 0)        # a test that failed mid-cycle must not leave the engine paused
+    for k, v in defaults.items():
+        assert fresh.amem_set_option(k, v) == 0
+
+
+def oracle_twin(orc, fp, caller=B.CALLER_P2P):
+    """The same footprint registered with the oracle, in its host-memory VMM."""
+    out = []
+    for i, sz in enumerate(fp.sizes):
+        va, h, asz = C.c_uint64(), C.c_uint64(), C.c_uint64()
+        assert orc.oracle_vmm_alloc(int(sz), C.byref(va), C.byref(h), C.byref(asz)) == 0
+        np.frombuffer((C.c_uint8 * int(sz)).from_address(va.value), dtype=np.uint8)[:] = fp.region_bytes(i)
+        assert orc.oracle_add_alloc_info(0, va.value, asz.value, B.TYPE_LOCAL, 0, h.value, -1, 0, 0, caller) == 0
+        out.append((va.value, asz.value))
+    return out
+
+
+def same_as_oracle(lib, orc, vas, twin):
+    """Region i of the engine (address vas[i]) against region i of the oracle (address twin[i][0]):
+    addresses and handle values differ between the two address spaces, everything else must not."""
+    etab, otab = H.region_table(lib, 0), O.region_table(orc, 0)
+    assert len(etab) == len(otab)
+    pairs = [(etab[int(v)], otab[t[0]]) for v, t in zip(vas, twin) if int(v) in etab or t[0] in otab]
+    assert len(pairs) == len(etab)
+    for e, o in pairs:
+        for f in ("alloc_sz", "tags", "type", "state", "refcount", "peers", "has_peer", "oos_flag", "dev", "shared_fd"):
+            assert e[f] == o[f], (f, e[f], o[f])
+        assert (e["handle"] == 0) == (o["handle"] == 0)
+        assert (e["cpu_addr"] == 0) == (o["cpu_addr"] == 0) or e["parked_bytes"] == 0
+    ec, oc = H.counters(lib), O.counters(orc, 0)
+    for k in ("release_local_cnt", "release_shadow_cnt", "offload_cnt", "alloc_bytes", "del_bytes", "pause_cnt",
+              "resume_cnt", "paused"):
+        assert ec[k] == oc[k], (k, ec[k], oc[k])
+    assert lib.amem_handle_count(0) == oc["handle_count"]
+
+
+@pytest.mark.parametrize("path", [0, 1])
+def test_config2_cycle_bit_exact_same_va_same_table(eng, fresh_orc, path):
+    """BASELINE config 2: 256 regions (128x4 + 96x2 + 32x16 MiB), half of the 64 KiB chunks zero."""
+    lib, orc = eng, fresh_orc
+    assert lib.amem_set_option(b"pause_path", path) == 0
+    fp = Footprint(2, 1, threads=16)
+    free0 = H.mem_free(lib)
+    regs = H.Regions(lib, fp)
+    twin = oracle_twin(orc, fp)
+    same = lambda: same_as_oracle(lib, orc, regs.va, twin)
+    same()
+    before = regs.table()
+    va_before = regs.va.copy()
+    free1 = H.mem_free(lib)
+    assert lib.amem_mem_pause(0, 0) == 0 and orc.oracle_mem_pause(0) == 0
+    same()
+    st = H.cycle_stats(lib)
+    assert st["footprint_bytes"] == fp.total_bytes == 1216 * MiB
+    assert st["zero_chunks"] == fp.zero_chunks() and st["total_chunks"] == fp.nchunks
+    assert st["parked_bytes"] == (fp.nchunks - fp.zero_chunks()) * CHUNK
+    assert (st["dma_bytes"] > 0) == (path == 1)
+    assert H.mem_free(lib) - free1 >= fp.total_bytes - 64 * MiB       # physical memory is gone ...
+    for va, t in H.region_table(lib, 0).items():
+        assert t["state"] == B.STATE_HOLE and t["handle"] == 0 and lib.amem_handle_lookup(0, before[va]["handle"]) == 0
+    assert lib.amem_check_paused(0) == 1
+    assert lib.amem_mem_resume(0, 0) == 0 and orc.oracle_mem_resume(0) == 0
+    assert abs(H.mem_free(lib) - free1) <= 64 * MiB                    # ... and back
+    same()
+    assert (regs.va == va_before).all()
+    assert regs.mismatched_bytes() == 0
+    after = regs.table()
+    assert H.compare_tables(before, after) == []
+    for va, t in after.items():
+        assert lib.amem_handle_lookup(0, t["handle"]) == va
+    regs.free()
+    assert lib.amem_region_count(0) == 0 and lib.amem_handle_count(0) == 0
+    assert lib.amem_pool_trim() > 0
+
+
+def test_repeated_cycles_with_writes_between(eng):
+    """BASELINE config 3 at 1 GiB: repeated cycles, 1 % of chunks rewritten in between,
+    including zero -> non-zero and non-zero -> zero flips."""
+    lib = eng
+    fp = Footprint(3, 2, byte_budget=1 << 30, threads=16)
+    regs = H.Regions(lib, fp)
+    assert lib.amem_set_option(b"verify", 1) == 0
+    flips = set()
+    for cycle in range(5):
+        mask_before = fp.mask.copy()
+        touched = fp.mutate(cycle)
+        regs.write_chunks(touched)
+        flips |= {(int(mask_before[c]), int(fp.mask[c])) for c in touched}
+        assert lib.amem_mem_pause(0, 0) == 0
+        st = H.cycle_stats(lib)
+        assert st["zero_chunks"] == fp.zero_chunks()
+        assert lib.amem_mem_resume(0, 0) == 0
+        assert H.cycle_stats(lib)["verify_mismatch"] == 0
+        assert regs.mismatched_bytes() == 0
+    assert (1, 0) in flips and (0, 1) in flips
+    c = H.counters(lib)
+    assert c["pause_cnt"] == c["resume_cnt"] == 5 and c["offload_cnt"] == 0
+    regs.free()
+
+
+@pytest.mark.parametrize("opts", [{"zero_elide": 0}, {"pause_path": 0, "dma_min_bytes": 128 << 10},
+                                  {"staging_bytes": 8 << 20}, {"resume_batch_bytes": 1},
+                                  {"staging_bytes": 1 << 20, "resume_batch_bytes": 1 << 40}])
+def test_option_paths_are_all_bit_exact(eng, opts):
+    lib = eng
+    for k, v in opts.items():
+        assert lib.amem_set_option(k.encode(), v) == 0
+    fp = Footprint(2, 5, max_regions=40, threads=8)          # 40 x 4 MiB
+    regs = H.Regions(lib, fp)
+    before = regs.table()
+    for _ in range(2):
+        assert lib.amem_mem_pause(0, 0) == 0
+        st = H.cycle_stats(lib)
+        if opts.get("zero_elide") == 0:
+            assert st["parked_bytes"] == fp.total_bytes
+        if "dma_min_bytes" in opts:
+            assert st["dma_bytes"] > 0 and st["kernel_bytes"] > 0 and st["dma_bytes"] + st["kernel_bytes"] == st["parked_bytes"]
+        if opts.get("staging_bytes") == 1 << 20:
+            assert st["kernel_bytes"] > 0                   # regions larger than a staging buffer go direct
+        assert lib.amem_mem_resume(0, 0) == 0
+        assert regs.mismatched_bytes() == 0
+    after = regs.table()
+    assert [d for d in H.compare_tables(before, after) if d[1] != "handle_gen"] == []
+    regs.free()
+
+
+def test_all_zero_and_tiny_footprints(eng):
+    lib = eng
+    va, h, asz = C.c_uint64(), C.c_uint64(), C.c_uint64()
+    assert lib.amem_vmm_alloc(2 * MiB, 0, C.byref(va), C.byref(h), C.byref(asz)) == 0
+    z = np.zeros(2 * MiB, dtype=np.uint8)
+    lib.amem_copy_to_device(va.value, z.ctypes.data, z.nbytes)
+    assert lib.amem_add_alloc_info(va.value, asz.value, 0, 0, h.value, -1, 0, None, 0) == 0
+    assert lib.amem_mem_pause(0, 0) == 0
+    st = H.cycle_stats(lib)
+    assert st["parked_bytes"] == 0 and st["zero_chunks"] == 32
+    assert lib.amem_mem_resume(0, 0) == 0
+    out = np.full(2 * MiB, 9, dtype=np.uint8)
+    lib.amem_copy_from_device(out.ctypes.data, va.value, out.nbytes)
+    assert not out.any()
+    # a single non-zero byte at the very end survives
+    z[-1] = 0xA5
+    lib.amem_copy_to_device(va.value, z.ctypes.data, z.nbytes)
+    assert lib.amem_mem_pause(0, 0) == 0 and H.cycle_stats(lib)["parked_bytes"] == CHUNK
+    assert lib.amem_mem_resume(0, 0) == 0
+    lib.amem_copy_from_device(out.ctypes.data, va.value, out.nbytes)
+    assert np.array_equal(out, z)
+    lib.amem_del_alloc_info(va.value, 0, 0)
+    lib.amem_vmm_free(va.value, asz.value, 0)
+
+
+def test_state_machine_edges(eng, fresh_orc):
+    """Idempotence, the paused gate, delete while paused, empty table (amem_nccl.cpp:481-493, :133-137, :589-594)."""
+    lib, orc = eng, fresh_orc
+    # pause with nothing tracked: context does not even exist -> no-op
+    assert lib.amem_mem_pause(0, 0) == 0 and lib.amem_check_paused(0) == 0
+    fp = Footprint(2, 9, max_regions=6, threads=4)
+    regs = H.Regions(lib, fp)
+    twin = oracle_twin(orc, fp)
+    same = lambda: same_as_oracle(lib, orc, regs.va, twin)
+    assert lib.amem_mem_resume(0, 0) == 0 and orc.oracle_mem_resume(0) == 0      # resume while not paused
+    same()
+    assert lib.amem_mem_pause(0, 0) == 0 and orc.oracle_mem_pause(0) == 0
+    assert lib.amem_mem_pause(0, 0) == 0 and orc.oracle_mem_pause(0) == 0        # second pause: no-op
+    same()
+    # the allocator hook is refused while paused
+    va, h, asz = C.c_uint64(), C.c_uint64(), C.c_uint64()
+    assert lib.amem_vmm_alloc(2 * MiB, 0, C.byref(va), C.byref(h), C.byref(asz)) == 0
+    assert lib.amem_add_alloc_info(va.value, asz.value, 0, 0, h.value, -1, 0, None, 1) == 1
+    assert orc.oracle_add_alloc_info(0, 0x1000, 2 * MiB, 0, 0, 5, -1, 0, 0, 1) == 1
+    assert lib.amem_vmm_free(va.value, asz.value, h.value) == 0
+    # a region deleted while paused stays a hole; the rest comes back
+    assert lib.amem_del_alloc_info(int(regs.va[2]), 0, 0) == 0 and orc.oracle_del_alloc_info(0, twin[2][0], 0, 0) == 0
+    assert lib.amem_mem_resume(0, 0) == 0 and orc.oracle_mem_resume(0) == 0
+    assert lib.amem_mem_resume(0, 0) == 0 and orc.oracle_mem_resume(0) == 0      # second resume: no-op
+    same()
+    assert lib.amem_vmm_free(int(regs.va[2]), int(regs.alloc[2]), 0) == 0          # only a reservation is left
+    keep = [i for i in range(len(regs.va)) if i != 2]
+    for i in keep:
+        buf = np.empty(int(fp.sizes[i]), dtype=np.uint8)
+        lib.amem_copy_from_device(buf.ctypes.data, int(regs.va[i]), buf.nbytes)
+        assert fp.check_region(i, buf) == 0
+    for i in keep:
+        lib.amem_del_alloc_info(int(regs.va[i]), 0, 0)
+        lib.amem_vmm_free(int(regs.va[i]), int(regs.alloc[i]), 0)
+    # ncclPause / ncclResume report success and do the same thing
+    regs2 = H.Regions(lib, Footprint(2, 10, max_regions=3, threads=2))
+    assert lib.ncclPause(None) == 0 and lib.amem_check_paused(0) == 1
+    assert lib.ncclResume(None) == 0 and lib.amem_check_paused(0) == 0
+    assert regs2.mismatched_bytes() == 0
+    regs2.free()
+
+
+def test_mixed_callers_and_sizes_not_chunk_multiples(eng):
+    """Regions whose size is a multiple of the 4 KiB VMM granularity but not of 64 KiB, registered
+    under several caller tags; a short last chunk must be saved and restored too."""
+    lib = eng
+    rng = np.random.default_rng(5)
+    items = []
+    for k, nbytes in enumerate([2 * MiB, 2 * MiB - 4096, 3 * CHUNK + 4096, 4096, 10 * MiB + 8192]):
+        va, h, asz = C.c_uint64(), C.c_uint64(), C.c_uint64()
+        assert lib.amem_vmm_alloc(nbytes, 0, C.byref(va), C.byref(h), C.byref(asz)) == 0
+        data = rng.integers(0, 256, nbytes, dtype=np.uint8)
+        data[nbytes // 2: nbytes // 2 + CHUNK] = 0
+        lib.amem_copy_to_device(va.value, data.ctypes.data, nbytes)
+        assert lib.amem_add_alloc_info(va.value, nbytes, 0, 0, h.value, -1, 0, None, (1, 3, 7, 0, 9)[k]) == 0
+        items.append((va.value, asz.value, nbytes, data))
+    c = H.counters(lib)
+    assert c["alloc_bytes"][1] == 2 * MiB and c["alloc_bytes"][9] == 10 * MiB + 8192
+    for _ in range(2):
+        assert lib.amem_mem_pause(0, 0) == 0 and lib.amem_mem_resume(0, 0) == 0
+    for va, asz, nbytes, data in items:
+        out = np.empty(nbytes, dtype=np.uint8)
+        lib.amem_copy_from_device(out.ctypes.data, va, nbytes)
+        assert np.array_equal(out, data)
+        lib.amem_del_alloc_info(va, 0, 0)
+        lib.amem_vmm_free(va, asz, 0)
+    assert H.counters(lib)["alloc_bytes"] == [0] * 16
+
+
+def test_full_size_headline_footprint_one_cycle(eng):
+    """The 10 GiB headline footprint (572 regions): one cycle, checked by regeneration."""
+    lib = eng
+    fp = Footprint(3, 2, byte_budget=10 << 30, threads=16)
+    regs = H.Regions(lib, fp)
+    before = regs.table()
+    free1 = H.mem_free(lib)
+    assert lib.amem_mem_pause(0, 0) == 0
+    assert H.mem_free(lib) - free1 >= fp.total_bytes - 256 * MiB
+    assert lib.amem_mem_resume(0, 0) == 0
+    st = H.cycle_stats(lib)
+    assert st["local_regions"] == 572 and st["total_chunks"] == fp.nchunks and st["zero_chunks"] == fp.zero_chunks()
+    assert regs.mismatched_bytes() == 0
+    assert H.compare_tables(before, regs.table()) == []
+    assert st["pause_ms"] + st["resume_ms"] < 1000.0          # the headline target: under one second
+    regs.free()

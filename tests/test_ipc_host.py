@@ -1,0 +1,72 @@
+"""Cross-process registration over the UNIX-socket service, without a GPU: an importer process
+tells the owner process which VA maps the owner's handle (reference: register_peer,
+gmm_client_impl.cpp:479-505 -> worker dispatch gmm_worker_impl.cpp:375-382 ->
+amem_registerPeerInfo, amem_nccl.cpp:297-329). Handles and addresses are made up; only the
+bookkeeping is exercised."""
+import ctypes as C
+import multiprocessing as mp
+import os
+import tempfile
+
+MiB = 1 << 20
+OWNER_VA, OWNER_HANDLE = 0x7f1000000000, 0xABCDE0
+
+
+def _owner(ipc_dir, gid, to_parent, from_parent):
+    os.environ.update(AMEM_ENABLE="1", GMM_LOG="1", GMM_IPC_DIR=ipc_dir, AMEM_GROUPID=str(gid))
+    from asystem_amem_amd import binding as B, harness as H
+    lib = B.load()
+    assert lib.amem_add_alloc_info(OWNER_VA, 4 * MiB, B.TYPE_LOCAL, 0, OWNER_HANDLE, -1, 0, None, B.CALLER_P2P) == 0
+    to_parent.send(("slot", lib.amem_get_slot()))
+    assert from_parent.recv() == "check"
+    t = H.region_table(lib, 0)[OWNER_VA]
+    to_parent.send(("table", t["has_peer"], t["peers"]))
+    assert from_parent.recv() == "exit"
+    lib.amem_shutdown()
+
+
+def _importer(ipc_dir, gid, owner_slot, to_parent, from_parent):
+    os.environ.update(AMEM_ENABLE="1", GMM_LOG="1", GMM_IPC_DIR=ipc_dir, AMEM_GROUPID=str(gid))
+    from asystem_amem_amd import binding as B, harness as H
+    lib = B.load()
+    lib.amem_set_option(b"peer_timeout_ms", 3000)
+    my_va = 0x7f2000000000
+    ok = lib.amem_add_alloc_info(my_va, 4 * MiB, B.TYPE_PEER_POSIX, 0, 0x111, owner_slot, OWNER_HANDLE, None,
+                                 B.CALLER_P2P_PEER)
+    bad = lib.amem_add_alloc_info(my_va + (1 << 30), 4 * MiB, B.TYPE_PEER_POSIX, 0, 0x112, owner_slot, 0xBAD, None,
+                                  B.CALLER_P2P_PEER)
+    nobody = lib.amem_add_alloc_info(my_va + (2 << 30), 4 * MiB, B.TYPE_PEER_POSIX, 0, 0x113, 6, OWNER_HANDLE, None,
+                                     B.CALLER_P2P_PEER)
+    to_parent.send(("result", lib.amem_get_slot(), ok, bad, nobody, sorted(H.region_table(lib, 0))))
+    assert from_parent.recv() == "exit"
+    lib.amem_shutdown()
+
+
+def test_register_peer_across_processes():
+    ctx = mp.get_context("spawn")
+    with tempfile.TemporaryDirectory() as ipc_dir:
+        gid = 0x5000 + os.getpid() % 4096
+        o_out, o_in = ctx.Pipe(), ctx.Pipe()
+        owner = ctx.Process(target=_owner, args=(ipc_dir, gid, o_out[1], o_in[0]))
+        owner.start()
+        tag, owner_slot = o_out[0].recv()
+        assert tag == "slot" and 0 <= owner_slot < 8
+        i_out, i_in = ctx.Pipe(), ctx.Pipe()
+        imp = ctx.Process(target=_importer, args=(ipc_dir, gid, owner_slot, i_out[1], i_in[0]))
+        imp.start()
+        assert i_out[0].poll(60)
+        tag, imp_slot, ok, bad, nobody, imp_table = i_out[0].recv()
+        assert imp_slot not in (-1, owner_slot)            # slots are claimed first-free
+        assert ok == 0                                     # owner knew the handle
+        assert bad == 1 and nobody == 1                    # unknown handle / no such owner: dropped
+        assert imp_table == [0x7f2000000000]               # only the good import stays in scope
+        o_in[1].send("check")
+        tag, has_peer, peers = o_out[0].recv()
+        assert has_peer == 1 and peers[imp_slot] == 0x7f2000000000
+        assert sum(1 for p in peers if p) == 1
+        i_in[1].send("exit")
+        o_in[1].send("exit")
+        imp.join(30)
+        owner.join(30)
+        assert imp.exitcode == 0 and owner.exitcode == 0
+        assert not [f for f in os.listdir(ipc_dir) if f.endswith(".sock")]   # sockets removed on shutdown
