@@ -77,6 +77,9 @@ def main():
     ap.add_argument("--gib", type=float, default=10.0, help="footprint budget in GiB (headline: 10)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pause-path", type=int, default=None)
+    ap.add_argument("--calib", action="store_true",
+                    help="also run the plain 1 GiB copy kernel once, so that a counter profile of this command "
+                         "holds a kernel of known HBM traffic (1 GiB read + 1 GiB written)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the pause/resume engine has no multi-GPU path "
@@ -96,6 +99,10 @@ def main():
 
     d2h, h2d = C.c_double(), C.c_double()
     assert lib.amem_probe_link(1 << 30, 3, C.byref(d2h), C.byref(h2d)) == 0
+
+    if args.calib:
+        ms = C.c_float()
+        assert lib.amem_calib_copy(1 << 30, 3, C.byref(ms)) == 0
 
     fp = Footprint(3, 2, byte_budget=int(args.gib * (1 << 30)), threads=host_threads)
     regs = H.Regions(lib, fp)
