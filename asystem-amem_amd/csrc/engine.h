@@ -27,6 +27,7 @@ struct Options {
   int64_t hbm_wgs = 8192;                 // workgroup cap of device-only kernels
   int64_t resume_batch_bytes = 64ll << 20;
   int64_t peer_timeout_ms = 60000;
+  int64_t peer_loopback = 0;              // let a process register with / update its own service (tests)
 };
 Options& options();
 

@@ -305,7 +305,7 @@ void ipc_stop() {
 }
 
 int peer_register(uint64_t src_handle, uint64_t my_va, int owner_slot) {
-  if (g_svc.slot < 0 || owner_slot == g_svc.slot) return 1;
+  if (g_svc.slot < 0 || (owner_slot == g_svc.slot && !options().peer_loopback)) return 1;
   WireReq req = {kMagic, OP_REGISTER_PEER_INFO, g_svc.slot, (int32_t)getpid(), src_handle, my_va};
   int ret = rpc(owner_slot, req, -1);
   if (ret != 0)
@@ -315,7 +315,7 @@ int peer_register(uint64_t src_handle, uint64_t my_va, int owner_slot) {
 }
 
 int peer_update(int importer_slot, uint64_t peer_va, int fd) {
-  if (importer_slot == g_svc.slot) return 0;
+  if (importer_slot == g_svc.slot && !options().peer_loopback) return 0;
   if (g_svc.slot < 0) return 1;
   WireReq req = {kMagic, OP_UPDATE_PEER_INFO, g_svc.slot, (int32_t)getpid(), 0, peer_va};
   int ret = rpc(importer_slot, req, fd);

@@ -266,7 +266,10 @@ int amem_set_enabled(int on);
  *   "staging_bytes"   size of each of the two device staging buffers
  *   "slab_bytes"      size of one pinned host slab (power of two)
  *   "link_wgs"        workgroups of a kernel that reads or writes host memory
- *   "peer_timeout_ms" how long resume waits for owners before failing (0 = forever) */
+ *   "peer_timeout_ms" how long resume waits for owners before failing (0 = forever)
+ *   "peer_loopback"   0/1   treat this process's own slot like any other peer: registration and
+ *                     re-export go through the socket service of the same process (default 0:
+ *                     a process never registers with itself, gmm_client_impl.cpp:482-484, :512-514) */
 int amem_set_option(const char* name, int64_t value);
 int64_t amem_get_option(const char* name);
 
