@@ -4,7 +4,9 @@
 #include <unistd.h>
 
 #include <algorithm>
+#include <atomic>
 #include <chrono>
+#include <thread>
 
 #include "ipc.h"
 #include "log.h"
@@ -370,6 +372,77 @@ hipError_t Engine::pause_copy_direct(Ctx& c, std::vector<Region*>& regs) {
   return e;
 }
 
+// Interleaved path: the gather kernel writes pinned host memory itself, in many short
+// launches (one per group of regions holding about interleave_bytes of parked data), with an
+// event after each. A second host thread unmaps and releases a group's regions as soon as
+// that group's event has fired. An unmap issued while kernels are queued waits for roughly
+// one kernel boundary, and the kernels keep running at link rate meanwhile, so short
+// launches let most of the unmap time hide behind the transfer; a copy-engine transfer
+// would instead stall for the whole of every unmap.
+hipError_t Engine::pause_copy_interleaved(Ctx& c, std::vector<Region*>& regs) {
+  hipError_t e;
+  uint64_t ntiles_all = 0;
+  if ((e = upload_descs(gather_descs_.data(), gather_descs_.size(), &ntiles_all)) != hipSuccess) return e;
+  const uint64_t* tp = (const uint64_t*)h_tiles_.p;
+  SlabTable pool_tab = {(uint8_t* const*)d_slabtab_.p, pool_->shift(), pool_->slab_bytes() - 1};
+  const uint64_t want = (uint64_t)std::max<int64_t>(options().interleave_bytes, (int64_t)kChunkBytes);
+  struct Group { size_t r0, r1; uint32_t d0, d1; uint64_t bytes; };
+  std::vector<Group> groups;
+  const size_t n = parked_.size();
+  for (size_t i = 0; i < n;) {
+    size_t j = i;
+    uint64_t bytes = 0;
+    while (j < n && (bytes < want || j == i)) bytes += parked_[j++].parked_bytes;
+    groups.push_back({i, j, parked_[i].desc_begin, parked_[j - 1].desc_end, bytes});
+    i = j;
+  }
+  const size_t ev0 = 8;
+  hipEvent_t start = event_at(ev0 + groups.size());  // creates every event before the thread starts
+  std::atomic<size_t> launched{0};
+  std::atomic<int> failed{0};
+  auto tc = Clock::now();
+  std::thread unmapper([&] {
+    (void)hipSetDevice(dev_);
+    for (size_t g = 0; g < groups.size(); ++g) {
+      while (launched.load(std::memory_order_acquire) <= g) {
+        if (failed.load()) return;
+        std::this_thread::yield();
+      }
+      if (hipEventSynchronize(events_[ev0 + g]) != hipSuccess) { failed.store((int)hipGetLastError()); return; }
+      for (size_t r = groups[g].r0; r < groups[g].r1; ++r) {
+        hipError_t e2 = release_local(c, regs[r], parked_[r].va);
+        if (e2 != hipSuccess) { failed.store((int)e2); return; }
+      }
+    }
+  });
+  (void)CHECK_HIP(hipEventRecord(start, kstream_));
+  e = hipSuccess;
+  for (size_t g = 0; g < groups.size(); ++g) {
+    const Group& G = groups[g];
+    if (G.d1 > G.d0 && tp[G.d1] > tp[G.d0]) {
+      e = CHECK_HIP(launch_move(false, (const CopyDesc*)d_descs_.p + G.d0, (const uint64_t*)d_tiles_.p + G.d0,
+                                G.d1 - G.d0, tp[G.d0], tp[G.d1] - tp[G.d0], pool_tab, 0,
+                                (uint32_t)options().link_wgs, kstream_));
+      if (e != hipSuccess) break;
+      stats_.k2_launches++;
+      stats_.kernel_bytes += G.bytes;
+    }
+    e = CHECK_HIP(hipEventRecord(events_[ev0 + g], kstream_));
+    if (e != hipSuccess) break;
+    launched.store(g + 1, std::memory_order_release);
+  }
+  if (e != hipSuccess) failed.store((int)e);
+  unmapper.join();
+  hipError_t es = CHECK_HIP(hipStreamSynchronize(kstream_));
+  stats_.pause_copy_ms = ms_since(tc);
+  if (!groups.empty()) {
+    float ms = 0;
+    if (hipEventElapsedTime(&ms, start, events_[ev0 + groups.size() - 1]) == hipSuccess) stats_.k2_ms += ms;
+  }
+  if (failed.load()) return (hipError_t)failed.load();
+  return es;
+}
+
 // Staged path: regions are taken in rounds that fit one device staging buffer. A round is
 // packed by a gather kernel at HBM rate, then leaves as a few large hipMemcpyAsync calls
 // while the host unmaps and releases that round's regions. No kernel is in flight while
@@ -386,7 +459,7 @@ hipError_t Engine::pause_copy_staged(Ctx& c, std::vector<Region*>& regs, bool* u
     void* p = nullptr;
     if (hipMalloc(&p, need) != hipSuccess) {
       (void)hipGetLastError();
-      LOGGER(INFO, "memPause: no room for %llu MiB of device staging, using the direct path",
+      LOGGER(INFO, "memPause: no room for %llu MiB of device staging, using the interleaved path",
              (unsigned long long)(need >> 20));
       d_staging_[0].release();
       d_staging_[1].release();
@@ -587,10 +660,18 @@ int Engine::pause(Ctx& c) {
   if (rc == 0) {
     bool staged = false;
     const int64_t path = options().pause_path;
-    if (path != 0 && !locals.empty()) note(pause_copy_staged(c, locals, &staged));
-    if (!staged && rc == 0) {
+    if (path == 3 && !locals.empty()) {
       note(upload_slab_table());
-      note(pause_copy_direct(c, locals));
+      note(pause_copy_interleaved(c, locals));
+      staged = true;
+    } else if (path != 0 && !locals.empty()) {
+      note(pause_copy_staged(c, locals, &staged));
+    }
+    if (!staged && rc == 0) {
+      // no room for device staging (or path 0 asked for): write host memory from the kernel
+      note(upload_slab_table());
+      if (path == 0) note(pause_copy_direct(c, locals));
+      else note(pause_copy_interleaved(c, locals));
     }
   }
   // The sums copy above rode kstream_; make sure it landed before the scratch is reused.

@@ -19,7 +19,8 @@ namespace amem {
 struct Options {
   int64_t zero_elide = 1;
   int64_t verify = 0;
-  int64_t pause_path = 2;                 // 0 direct, 1 staged, 2 auto
+  int64_t pause_path = 2;                 // 0 direct, 1 staged, 2 auto, 3 interleaved
+  int64_t interleave_bytes = 8ll << 20;   // interleaved path: parked bytes per gather launch
   int64_t dma_min_bytes = 16ll << 20;     // direct path: runs this long go by hipMemcpyAsync
   int64_t staging_bytes = 256ll << 20;    // each of two device staging buffers
   int64_t slab_bytes = 256ll << 20;
@@ -85,6 +86,7 @@ class Engine {
   hipError_t upload_slab_table();
   hipError_t pause_copy_direct(Ctx& c, std::vector<Region*>& regs);
   hipError_t pause_copy_staged(Ctx& c, std::vector<Region*>& regs, bool* used);
+  hipError_t pause_copy_interleaved(Ctx& c, std::vector<Region*>& regs);
   hipError_t release_local(Ctx& c, Region* r, uint64_t va);
   hipEvent_t event_at(size_t i);
 

@@ -77,6 +77,7 @@ def main():
     ap.add_argument("--gib", type=float, default=10.0, help="footprint budget in GiB (headline: 10)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pause-path", type=int, default=None)
+    ap.add_argument("--opt", action="append", default=[], help="engine tunable, name=value (see amem_set_option)")
     ap.add_argument("--calib", action="store_true",
                     help="also run the plain 1 GiB copy kernel once, so that a counter profile of this command "
                          "holds a kernel of known HBM traffic (1 GiB read + 1 GiB written)")
@@ -95,6 +96,9 @@ def main():
         sys.exit("bench.py needs a GPU")
     if args.pause_path is not None:
         lib.amem_set_option(b"pause_path", args.pause_path)
+    for kv in args.opt:
+        k, v = kv.split("=")
+        assert lib.amem_set_option(k.encode(), int(v)) == 0, kv
     host_threads = min(16, os.cpu_count() or 1)
 
     d2h, h2d = C.c_double(), C.c_double()

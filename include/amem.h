@@ -259,9 +259,12 @@ int amem_set_enabled(int on);
 /* Tunables. Unknown name or bad value returns 1. Names:
  *   "zero_elide"      0/1   skip all-zero 64 KiB chunks (default 1)
  *   "verify"          0/1   re-scan after resume and compare checksums (default 0)
- *   "pause_path"      0 = pack kernel writes pinned host memory directly,
- *                     1 = pack into device staging, then large hipMemcpyAsync, unmap overlapped
- *                     2 = choose 1 when staging memory can be allocated, else 0 (default)
+ *   "pause_path"      0 = one pack kernel writes pinned host memory, then regions are unmapped
+ *                     1 = pack into device staging, large hipMemcpyAsync, unmap during the transfer
+ *                     2 = 1 when staging memory can be allocated, else 3 (default)
+ *                     3 = many short pack launches into pinned host memory, a second host
+ *                         thread unmaps each group of regions as soon as its launch is done
+ *   "interleave_bytes" parked bytes per launch of path 3
  *   "dma_min_bytes"   extents at least this long use hipMemcpyAsync in the direct path
  *   "staging_bytes"   size of each of the two device staging buffers
  *   "slab_bytes"      size of one pinned host slab (power of two)

@@ -131,6 +131,33 @@ def test_region_order_and_find(fresh):
     assert lib.amem_region_count(5) == 0
 
 
+def test_registry_latency_with_100k_entries(fresh):
+    """The registry side of BASELINE config 4: 100,000 entries inserted, looked up and deleted.
+    The bound is loose (shared CI cores); the measured figure is printed."""
+    import time
+    lib = fresh
+    n = 100000
+    base = 0x7e0000000000
+    lib.amem_add_alloc_info(base - 4096, 4096, 0, 0, 1, -1, 0, None, 1)   # first add: starts the socket service
+    t0 = time.perf_counter()
+    for i in range(n):
+        lib.amem_add_alloc_info(base + i * 65536, 4096 * (1 + i % 16), 0, 0, 0x100000 + i, -1, 0, None, 1)
+    t1 = time.perf_counter()
+    assert lib.amem_region_count(0) == n + 1 and lib.amem_handle_count(0) == n + 1
+    info = B.RegionInfo()
+    for i in range(0, n, 7):
+        assert lib.amem_region_find(0, base + i * 65536, C.byref(info)) == 0 and info.handle == 0x100000 + i
+    t2 = time.perf_counter()
+    for i in range(n):
+        lib.amem_del_alloc_info(base + i * 65536, 0x100000 + i, 0)
+    t3 = time.perf_counter()
+    assert lib.amem_region_count(0) == 1 and lib.amem_handle_count(0) == 1
+    add_us, find_us, del_us = (t1 - t0) / n * 1e6, (t2 - t1) / (n / 7) * 1e6, (t3 - t2) / n * 1e6
+    print("registry latency with 100k entries, including the ctypes call: add %.2f us, find %.2f us, del %.2f us"
+          % (add_us, find_us, del_us))
+    assert add_us < 50 and find_us < 50 and del_us < 50
+
+
 def test_disabled_engine_ignores_everything(fresh):
     lib = fresh
     assert lib.amem_set_enabled(0) == 0

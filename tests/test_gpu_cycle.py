@@ -56,7 +56,7 @@ def same_as_oracle(lib, orc, vas, twin):
     assert lib.amem_handle_count(0) == oc["handle_count"]
 
 
-@pytest.mark.parametrize("path", [0, 1])
+@pytest.mark.parametrize("path", [0, 1, 3])
 def test_config2_cycle_bit_exact_same_va_same_table(eng, fresh_orc, path):
     """BASELINE config 2: 256 regions (128x4 + 96x2 + 32x16 MiB), half of the 64 KiB chunks zero."""
     lib, orc = eng, fresh_orc

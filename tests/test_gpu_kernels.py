@@ -168,38 +168,47 @@ def test_pack_unpack_match_oracle(gpu, orc, host_side):
         stage.free()
 
 
-def test_fragmented_descriptor_list_round_trip(gpu, orc):
-    """The shape of BASELINE config 4 at 1/50 scale: 2,000 sub-allocations of 4-64 KiB bump-packed
-    into 2 MiB granules, gathered into contiguous staging and scattered back into fresh memory."""
-    fp = Footprint(4, 3, max_regions=2000)
+@pytest.mark.parametrize("count", [2000, 100000])
+def test_fragmented_descriptor_list_round_trip(gpu, orc, count):
+    """BASELINE config 4 (100,000 sub-allocations of 4-64 KiB bump-packed into 2 MiB granules, seed 3;
+    also at 1/50 scale): gathered into contiguous staging and scattered back into fresh memory."""
+    fp = Footprint(4, 3, max_regions=count, threads=16)
     granule = 2 * MiB
-    placements, cur = [], 0
-    for sz in fp.sizes:                                  # bump allocation, no sub-allocation straddles a granule
-        sz = int(sz)
+    sizes = fp.sizes.astype(np.int64)
+    starts = np.zeros(len(sizes), dtype=np.int64)
+    cur = 0
+    for i, sz in enumerate(sizes):                       # bump allocation, no sub-allocation straddles a granule
         if cur % granule + sz > granule:
             cur = (cur // granule + 1) * granule
-        placements.append((cur, sz))
+        starts[i] = cur
         cur += sz
-    total = (cur + granule - 1) // granule * granule
+    total = int((cur + granule - 1) // granule * granule)
     src, dst = DevBuf(gpu, total), DevBuf(gpu, total)
     host = np.zeros(total, dtype=np.uint8)
-    for i, (a, n) in enumerate(placements):
-        host[a:a + n] = fp.region_bytes(i)
+    for i in range(len(sizes)):
+        fp.region_bytes(i, host[starts[i]:starts[i] + sizes[i]])
     src.put(host)
     dst.put(np.full(total, 0x77, dtype=np.uint8))
-    packed = int(fp.sizes.sum())
+    packed = int(sizes.sum())
     stage = DevBuf(gpu, packed)
-    offs = np.concatenate([[0], np.cumsum(fp.sizes)]).astype(np.uint64)
-    g = _descs([(src.va + a, int(offs[i]), n) for i, (a, n) in enumerate(placements)])
-    assert gpu.amem_gather_pack(g, len(placements), stage.va, packed, 0, None) == 0
-    want = np.concatenate([host[a:a + n] for a, n in placements])
-    assert np.array_equal(stage.get(packed), want)
-    s = _descs([(dst.va + a, int(offs[i]), n) for i, (a, n) in enumerate(placements)])
-    assert gpu.amem_scatter_unpack(s, len(placements), stage.va, packed, 0, None) == 0
-    back = dst.get(total)
+    offs = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+    garr = np.empty((len(sizes), 3), dtype=np.uint64)
+    garr[:, 0] = src.va + starts
+    garr[:, 1] = offs[:-1]
+    garr[:, 2] = sizes
+    ms = C.c_float()
+    assert gpu.amem_gather_pack(garr.ctypes.data_as(C.POINTER(B.CopyDesc)), len(sizes), stage.va, packed, 0, C.byref(ms)) == 0
     live = np.zeros(total, dtype=bool)
-    for a, n in placements:
+    idx = np.concatenate([np.arange(a, a + n) for a, n in zip(starts[:4000], sizes[:4000])])   # spot-check layout
+    got = stage.get(packed)
+    assert np.array_equal(got[:len(idx)], host[idx])
+    for a, n in zip(starts, sizes):
         live[a:a + n] = True
+    assert np.array_equal(got, host[live])              # packed order == address order for a bump allocator
+    sarr = garr.copy()
+    sarr[:, 0] = dst.va + starts
+    assert gpu.amem_scatter_unpack(sarr.ctypes.data_as(C.POINTER(B.CopyDesc)), len(sizes), stage.va, packed, 0, C.byref(ms)) == 0
+    back = dst.get(total)
     assert np.array_equal(back[live], host[live]) and (back[~live] == 0x77).all()
     src.free(); dst.free(); stage.free()
 
