@@ -209,6 +209,7 @@ int amem_add_alloc_info(uint64_t va, uint64_t size, int type, int dev, uint64_t 
   } else if (!peerFlag) {
     // Case 4: local memory is indexed by handle (amem_nccl.cpp:258-265).
     std::lock_guard<std::mutex> ls(c->structure);
+    std::lock_guard<std::mutex> lf(c->fields);   // the service thread looks handles up under `fields`
     c->handleTable[dev].emplace(handle, va);
   }
   {

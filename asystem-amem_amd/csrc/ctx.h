@@ -47,8 +47,9 @@ static inline bool from_peer(int type) { return type > AMEM_TYPE_LOCAL_SYMM; }  
 struct Ctx {
   // `structure` guards insertion and erasure in the tables and is held for the whole of a
   // pause or resume, so the engine may keep pointers to map nodes. `fields` guards region
-  // fields and counters that the IPC service thread also touches (peers[], hasPeer, state
-  // of imported regions, releaseShadowCnt). Lock order: structure, then fields.
+  // fields, counters and the handle index, which the IPC service thread also touches (peers[],
+  // hasPeer, state of imported regions, releaseShadowCnt, handleTable lookups): readers hold
+  // `fields`, writers of the tables hold both. Lock order: structure, then fields.
   std::mutex structure;
   std::mutex fields;
   std::condition_variable shadow_cv;  // signalled when releaseShadowCnt drops

@@ -323,8 +323,8 @@ hipError_t Engine::release_local(Ctx& c, Region* r, uint64_t va) {
     c.releaseLocalCnt += popcount_peers(*r);
     r->state = AMEM_STATE_HOLE;
     r->handle = 0;
+    c.handleTable[dev_].erase(old);
   }
-  c.handleTable[dev_].erase(old);
   stats_.pause_unmap_ms += ms_since(t0);
   return e;
 }
@@ -796,6 +796,7 @@ int Engine::resume(Ctx& c) {
         im.r->handle = newh;  // amem_updateAllocInfo, amem_nccl.cpp:272-291
         im.r->handleGen++;
         has_peer = im.r->hasPeer;
+        c.handleTable[dev_].emplace(newh, im.va);
       }
       if (has_peer) {
         int fd = -1;
@@ -803,7 +804,6 @@ int Engine::resume(Ctx& c) {
         exports.push_back({im.r, im.va, fd});
         exportSz += im.r->allocSz;
       }
-      c.handleTable[dev_].emplace(newh, im.va);
       bytes += im.bytes;
       ++j;
     }

@@ -204,3 +204,30 @@ def test_missing_library_is_an_error(monkeypatch):
     with pytest.raises(RuntimeError):
         B.load("/nonexistent/libamem_nccl.so.1")
     monkeypatch.undo()
+
+
+def test_memstats_output_matches_readme_sample():
+    """ncclMemStats() prints per-caller bytes and the total (DEBUG level, amem_nccl.cpp:82-99). Fed with the
+    byte counts of the sample in the reference's README.md:206-211 it must print the README's total."""
+    import json
+    import sys
+    g = json.load(open(os.path.join(ROOT, "tests", "golden", "memstats_readme.json")))
+    code = (
+        "import ctypes, os, sys\n"
+        "sys.path.insert(0, %r)\n"
+        "from asystem_amem_amd import binding as B\n"
+        "lib = B.load()\n"
+        "va = 0x7f0000000000\n"
+        "for caller, n in %r.items():\n"
+        "    assert lib.amem_add_alloc_info(va, n, 0, 0, va + 1, -1, 0, None, int(caller)) == 0\n"
+        "    va += 1 << 36\n"
+        "assert lib.ncclMemStats() == 0\n"
+        "lib.amem_shutdown()\n" % (ROOT, g["caller_bytes"]))
+    env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="4", AMEM_GROUPID="170", AMEM_IPC="0")
+    out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, check=True).stdout
+    lines = [l for l in out.splitlines() if "DumpStats" in l]
+    for caller, n in g["caller_bytes"].items():
+        assert any("groupID:170" in l and ("caller_%s allocBytes:%d" % (caller, n)) in l for l in lines), lines
+    total = [l for l in lines if "in total" in l]
+    assert len(total) == 1 and ("total GPU alloc:%d (%d MB)" % (g["total_bytes"], g["total_mb"])) in total[0]
+    assert all(l.startswith("AMEM [DEBG] capi.cpp:amem_dump_alloc_stats:") for l in lines)   # the reference's line format

@@ -288,3 +288,47 @@ def test_peer_path_in_loopback(gpu, fresh):
     finally:
         lib.amem_mem_resume(0, 0)
         assert lib.amem_set_option(b"peer_loopback", 0) == 0
+
+
+def test_importer_times_out_when_owner_never_re_exports(gpu, fresh):
+    """Failure handling the reference lacks (its resume spins forever, amem_nccl.cpp:659-662): an
+    importer whose owner forgot the region before resume gives up after peer_timeout_ms, reports
+    an error and stays consistent. Forced from the host: nothing on the GPU hangs or faults."""
+    from asystem_amem_amd import binding as B, harness as H
+    from asystem_amem_amd.footprint import Footprint
+    lib = fresh
+    old_to = lib.amem_get_option(b"peer_timeout_ms")
+    assert lib.amem_set_option(b"peer_loopback", 1) == 0 and lib.amem_set_option(b"peer_timeout_ms", 300) == 0
+    try:
+        fp = Footprint(2, 12, max_regions=2, threads=2)
+        regs = H.Regions(lib, fp)
+        slot = lib.amem_get_slot()
+        fd, va, h = C.c_int(-1), C.c_uint64(), C.c_uint64()
+        assert lib.amem_vmm_export(int(regs.handle[0]), C.byref(fd)) == 0
+        assert lib.amem_vmm_import(fd.value, int(regs.alloc[0]), 0, C.byref(va), C.byref(h)) == 0
+        os.close(fd.value)
+        assert lib.amem_add_alloc_info(va.value, int(regs.alloc[0]), B.TYPE_PEER_POSIX, 0, h.value, slot,
+                                       int(regs.handle[0]), None, B.CALLER_P2P_PEER) == 0
+        # the "owner" drops its record of region 0: nobody will re-export it
+        assert lib.amem_del_alloc_info(int(regs.va[0]), int(regs.handle[0]), 0) == 0
+        assert lib.amem_mem_pause(0, 0) == 0
+        assert H.counters(lib)["release_shadow_cnt"] == 1
+        t0 = time.perf_counter()
+        rc = lib.amem_mem_resume(0, 0)
+        waited = time.perf_counter() - t0
+        assert rc != 0 and 0.25 < waited < 5.0
+        c = H.counters(lib)
+        assert c["paused"] == 0 and c["release_shadow_cnt"] == 1            # reported, not hidden
+        assert H.region_table(lib, 0)[va.value]["state"] == B.STATE_HOLE    # the orphaned import is still a hole
+        buf = np.empty(int(fp.sizes[1]), dtype=np.uint8)                    # everything else came back
+        assert lib.amem_copy_from_device(buf.ctypes.data, int(regs.va[1]), buf.nbytes) == 0
+        assert fp.check_region(1, buf) == 0
+        lib.amem_del_alloc_info(va.value, 0, 0)
+        lib.amem_vmm_free(va.value, int(regs.alloc[0]), 0)
+        lib.amem_vmm_free(int(regs.va[0]), int(regs.alloc[0]), 0)          # still mapped: it was never paused
+        lib.amem_del_alloc_info(int(regs.va[1]), 0, 0)
+        lib.amem_vmm_free(int(regs.va[1]), int(regs.alloc[1]), 0)
+    finally:
+        lib.amem_mem_resume(0, 0)
+        lib.amem_set_option(b"peer_loopback", 0)
+        lib.amem_set_option(b"peer_timeout_ms", old_to)

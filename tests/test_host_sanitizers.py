@@ -1,0 +1,56 @@
+"""The host side of the library under ThreadSanitizer and AddressSanitizer (the reference has no
+sanitizer runs and leaves its registry unguarded against its own worker thread,
+amem_nccl.cpp:303, :342, :365, :391). The library's own sources are rebuilt with the sanitizer on
+the host pass only and linked with tests/host_race/registry_hammer.cpp; nothing touches a GPU."""
+import os
+import shutil
+import subprocess
+import tempfile
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "asystem-amem_amd", "csrc")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+SOURCES = ["capi.cpp", "engine.cpp", "ipc.cpp", "log.cpp", "slab_pool.cpp", "vmm.cpp"]
+
+
+def build(kind, outdir):
+    san = ["-Xarch_host", "-fsanitize=" + kind]
+    common = ["-O1", "-g", "-std=c++17", "-fPIC", "-D__HIP_PLATFORM_AMD__", "-fno-omit-frame-pointer"]
+    objs = []
+    for src in SOURCES:
+        obj = os.path.join(outdir, src + "." + kind + ".o")
+        subprocess.run([HIPCC] + common + san + ["-c", os.path.join(CSRC, src), "-o", obj], check=True,
+                       capture_output=True, text=True)
+        objs.append(obj)
+    kobj = os.path.join(outdir, "kernels." + kind + ".o")
+    subprocess.run([HIPCC] + common + san + ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+                   "-packed-fp32-ops", "-c", os.path.join(CSRC, "kernels.hip"), "-o", kobj], check=True,
+                   capture_output=True, text=True)
+    hobj = os.path.join(outdir, "hammer." + kind + ".o")
+    subprocess.run([HIPCC] + common + san + ["-c", os.path.join(ROOT, "tests", "host_race", "registry_hammer.cpp"),
+                   "-o", hobj], check=True, capture_output=True, text=True)
+    exe = os.path.join(outdir, "hammer_" + kind)
+    subprocess.run([HIPCC] + san + ["--offload-arch=gfx950", hobj, kobj] + objs + ["-o", exe, "-lpthread"],
+                   check=True, capture_output=True, text=True)
+    return exe
+
+
+@pytest.mark.parametrize("kind", ["thread", "address"])
+def test_registry_hammer_under_sanitizer(kind):
+    if not os.path.exists(HIPCC):
+        pytest.skip("hipcc not found")
+    outdir = tempfile.mkdtemp(prefix="amem_san_")
+    try:
+        exe = build(kind, outdir)
+        env = dict(os.environ, GMM_LOG="1", GMM_IPC_DIR=outdir, AMEM_GROUPID=str(0x7000 + os.getpid() % 1000),
+                   TSAN_OPTIONS="exitcode=66 halt_on_error=0 report_signal_unsafe=0",
+                   ASAN_OPTIONS="exitcode=67 detect_leaks=0 protect_shadow_gap=0")
+        r = subprocess.run([exe], env=env, capture_output=True, text=True, timeout=180)
+        report = (r.stdout + r.stderr)[-6000:]
+        assert r.returncode == 0, report
+        assert "hammer done: 0 errors" in r.stdout, report
+        assert "WARNING: ThreadSanitizer" not in r.stderr and "ERROR: AddressSanitizer" not in r.stderr, report
+    finally:
+        shutil.rmtree(outdir, ignore_errors=True)
