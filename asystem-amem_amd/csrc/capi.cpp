@@ -575,7 +575,7 @@ static OptRef* opt_table(size_t* n) {
   static OptRef t[] = {
       {"zero_elide", &o.zero_elide, 0, 1},
       {"verify", &o.verify, 0, 1},
-      {"pause_path", &o.pause_path, 0, 3},
+      {"pause_path", &o.pause_path, 0, 4},
       {"interleave_bytes", &o.interleave_bytes, 1 << 16, (int64_t)1 << 40},
       {"dma_min_bytes", &o.dma_min_bytes, 0, (int64_t)1 << 40},
       {"staging_bytes", &o.staging_bytes, 0, (int64_t)1 << 36},

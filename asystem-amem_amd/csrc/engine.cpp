@@ -329,6 +329,33 @@ hipError_t Engine::release_local(Ctx& c, Region* r, uint64_t va) {
   return e;
 }
 
+// Reference structure, kept for A/B measurement only (pause_path 4): what amem_memPause does
+// (amem_nccl.cpp:502-513, :529-558) expressed in HIP calls — per region one whole-region
+// hipMemcpyAsync that is waited for before the next one starts, no scan, no elision; then per
+// region the handle is looked up from the mapping, unmapped and released.
+hipError_t Engine::pause_copy_reference(Ctx& c, std::vector<Region*>& regs) {
+  hipError_t e = hipSuccess;
+  auto tc = Clock::now();
+  for (size_t i = 0; i < regs.size(); ++i) {
+    for (uint32_t d = parked_[i].desc_begin; d < parked_[i].desc_end; ++d) {
+      const CopyDesc& cd = gather_descs_[d];
+      e = CHECK_HIP(hipMemcpyAsync(pool_->host_addr(cd.off), (const void*)(uintptr_t)cd.va, cd.bytes,
+                                   hipMemcpyDeviceToHost, dstream_));
+      if (e != hipSuccess) return e;
+      stats_.dma_bytes += cd.bytes;
+    }
+    e = CHECK_HIP(hipStreamSynchronize(dstream_));
+    if (e != hipSuccess) return e;
+  }
+  stats_.pause_copy_ms = ms_since(tc);
+  for (size_t i = 0; i < regs.size(); ++i) {
+    (void)vmm_handle_of(parked_[i].va);  // the reference's retain-to-discover (amem_nccl.cpp:539)
+    hipError_t e2 = release_local(c, regs[i], parked_[i].va);
+    if (e == hipSuccess) e = e2;
+  }
+  return e;
+}
+
 // Direct path: one gather kernel writes pinned host memory; runs of at least
 // dma_min_bytes go by hipMemcpyAsync on the second stream at the same time.
 hipError_t Engine::pause_copy_direct(Ctx& c, std::vector<Region*>& regs) {
@@ -564,7 +591,10 @@ int Engine::pause(Ctx& c) {
   if (e != hipSuccess) return (int)e;
   int rc = 0;
   auto note = [&](hipError_t x) { if (x != hipSuccess && rc == 0) rc = (int)x; };
-  const bool elide = options().zero_elide != 0;
+  const int64_t path = options().pause_path;
+  ref_mode_ = (path == 4);
+  const bool elide = options().zero_elide != 0 && !ref_mode_;
+  elide_used_ = elide;
   amem_cycle_stats fresh = {};
   fresh.slab_bytes = stats_.slab_bytes;
   stats_ = fresh;
@@ -614,21 +644,31 @@ int Engine::pause(Ctx& c) {
   }
   auto ts = Clock::now();
   float k1ms = 0;
-  have_sums_ = true;
-  e = run_scan(segs_, &nchunks_, true, &k1ms);
+  have_sums_ = !ref_mode_;
+  if (ref_mode_) {
+    // reference structure: no scan, every byte of every region is copied
+    nchunks_ = 0;
+    for (const ScanSeg& sg : segs_) nchunks_ += chunks_of(sg.bytes);
+    e = hipSuccess;
+  } else {
+    e = run_scan(segs_, &nchunks_, true, &k1ms);
+  }
   note(e);
-  if (e == hipSuccess && nchunks_) {
+  if (e == hipSuccess && nchunks_ && !ref_mode_) {
     note(h_sums_.ensure(nchunks_ * sizeof(ChunkSum)));
     note(CHECK_HIP(hipMemcpyAsync(h_sums_.p, d_sums_.p, nchunks_ * sizeof(ChunkSum), hipMemcpyDeviceToHost, kstream_)));
   }
   stats_.k1_ms = k1ms;
-  stats_.k1_launches = nchunks_ ? 1 : 0;
+  stats_.k1_launches = (nchunks_ && !ref_mode_) ? 1 : 0;
   stats_.pause_scan_ms = ms_since(ts);
+  // the flags drive resume; keep them where no later scan can overwrite them
+  if (ref_mode_) parked_flags_.assign(nchunks_, 0);
+  else parked_flags_.assign((const uint8_t*)h_flags_.p, (const uint8_t*)h_flags_.p + nchunks_);
   stats_.total_chunks = nchunks_;
 
   auto tp = Clock::now();
   uint64_t cursor = 0, chunk0 = 0, zero_chunks = 0;
-  const uint8_t* flags = (const uint8_t*)h_flags_.p;
+  const uint8_t* flags = parked_flags_.data();
   uint64_t slab_bytes = pool_->slab_bytes();
   for (size_t i = 0; i < locals.size(); ++i) {
     ParkedRegion p = {};
@@ -659,8 +699,10 @@ int Engine::pause(Ctx& c) {
 
   if (rc == 0) {
     bool staged = false;
-    const int64_t path = options().pause_path;
-    if (path == 3 && !locals.empty()) {
+    if (ref_mode_) {
+      note(pause_copy_reference(c, locals));
+      staged = true;
+    } else if (path == 3 && !locals.empty()) {
       note(upload_slab_table());
       note(pause_copy_interleaved(c, locals));
       staged = true;
@@ -715,7 +757,7 @@ int Engine::resume(Ctx& c) {
   if (e != hipSuccess) return (int)e;
   int rc = 0;
   auto note = [&](hipError_t x) { if (x != hipSuccess && rc == 0) rc = (int)x; };
-  const bool elide = options().zero_elide != 0;
+  const bool elide = elide_used_;
   size_t free_sz = 0, total = 0;
   (void)CHECK_HIP(hipMemGetInfo(&free_sz, &total));
   LOGGER(INFO, "groupID:%d pid:%d GPU:%d memUsed:%ld MB before resumed", amem_groupID_value(), getpid(), dev_,
@@ -729,7 +771,7 @@ int Engine::resume(Ctx& c) {
   struct Item { Region* r; uint64_t va; uint32_t d0, d1; uint64_t bytes; };
   std::vector<Item> items;
   std::vector<CopyDesc> scatter;
-  const uint8_t* flags = (const uint8_t*)h_flags_.p;
+  const uint8_t* flags = parked_flags_.data();
   const uint64_t slab_bytes = pool_->slab_bytes();
   std::vector<ScanSeg> verify_segs;
   std::vector<uint64_t> verify_first_chunk;
@@ -804,13 +846,23 @@ int Engine::resume(Ctx& c) {
         exports.push_back({im.r, im.va, fd});
         exportSz += im.r->allocSz;
       }
+      if (ref_mode_) {
+        // amem_lauchPreload with async=false (amem_nccl.h:316-327, call site amem_nccl.cpp:622):
+        // one copy per region, waited for before the next region is touched
+        for (uint32_t d = im.d0; d < im.d1; ++d) {
+          if (scatter[d].off == kDescZero) continue;
+          note(CHECK_HIP(hipMemcpyAsync((void*)(uintptr_t)scatter[d].va, pool_->host_addr(scatter[d].off), scatter[d].bytes,
+                                        hipMemcpyHostToDevice, dstream_)));
+        }
+        note(CHECK_HIP(hipStreamSynchronize(dstream_)));
+      }
       bytes += im.bytes;
       ++j;
     }
     stats_.resume_map_ms += ms_since(tm);
     if (j == i) break;
     const uint32_t d0 = items[i].d0, d1 = items[j - 1].d1;
-    if (d1 > d0 && tp[d1] > tp[d0]) {
+    if (!ref_mode_ && d1 > d0 && tp[d1] > tp[d0]) {
       hipEvent_t s0 = event_at(ev++), s1 = event_at(ev++);
       (void)CHECK_HIP(hipEventRecord(s0, kstream_));
       note(CHECK_HIP(launch_move(true, (const CopyDesc*)d_descs_.p + d0, (const uint64_t*)d_tiles_.p + d0,

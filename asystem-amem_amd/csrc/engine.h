@@ -19,7 +19,7 @@ namespace amem {
 struct Options {
   int64_t zero_elide = 1;
   int64_t verify = 0;
-  int64_t pause_path = 2;                 // 0 direct, 1 staged, 2 auto, 3 interleaved
+  int64_t pause_path = 2;                 // 0 direct, 1 staged, 2 auto, 3 interleaved, 4 reference structure (A/B only)
   int64_t interleave_bytes = 8ll << 20;   // interleaved path: parked bytes per gather launch
   int64_t dma_min_bytes = 16ll << 20;     // direct path: runs this long go by hipMemcpyAsync
   int64_t staging_bytes = 256ll << 20;    // each of two device staging buffers
@@ -87,6 +87,7 @@ class Engine {
   hipError_t pause_copy_direct(Ctx& c, std::vector<Region*>& regs);
   hipError_t pause_copy_staged(Ctx& c, std::vector<Region*>& regs, bool* used);
   hipError_t pause_copy_interleaved(Ctx& c, std::vector<Region*>& regs);
+  hipError_t pause_copy_reference(Ctx& c, std::vector<Region*>& regs);
   hipError_t release_local(Ctx& c, Region* r, uint64_t va);
   hipEvent_t event_at(size_t i);
 
@@ -109,6 +110,9 @@ class Engine {
   uint64_t nchunks_ = 0;
   uint64_t parked_total_ = 0;
   bool have_sums_ = false;
+  bool elide_used_ = true;   // zero_elide as it was when the parked layout was made
+  bool ref_mode_ = false;    // the parked layout was made by the reference-structure path
+  std::vector<uint8_t> parked_flags_;  // per-chunk zero flags of the last pause
 
   amem_cycle_stats stats_ = {};
 };

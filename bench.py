@@ -76,6 +76,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--gib", type=float, default=10.0, help="footprint budget in GiB (headline: 10)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-reference-structure", action="store_true")
     ap.add_argument("--pause-path", type=int, default=None)
     ap.add_argument("--opt", action="append", default=[], help="engine tunable, name=value (see amem_set_option)")
     ap.add_argument("--calib", action="store_true",
@@ -114,22 +115,42 @@ def main():
     va_before = regs.va.copy()
     table_before = regs.table()
 
-    pause_s, resume_s, stats = [], [], []
-    for step in range(args.warmup + args.steps):
-        touched = fp.mutate(step)  # writes between cycles, outside the clock
-        regs.write_chunks(touched)
-        t0 = time.perf_counter()
-        rc1 = lib.amem_mem_pause(0, 0)
-        t1 = time.perf_counter()
-        rc2 = lib.amem_mem_resume(0, 0)
-        t2 = time.perf_counter()
-        assert rc1 == 0 and rc2 == 0, (rc1, rc2)
-        if step >= args.warmup:
-            pause_s.append(t1 - t0)
-            resume_s.append(t2 - t1)
-            stats.append(H.cycle_stats(lib))
-        elif step == 0:
-            first = (t1 - t0, t2 - t1)
+    cycle_no = [0]
+
+    def run_cycles(warmup, steps):
+        pause_s, resume_s, stats, first = [], [], [], None
+        for step in range(warmup + steps):
+            touched = fp.mutate(cycle_no[0])  # writes between cycles, outside the clock
+            cycle_no[0] += 1
+            regs.write_chunks(touched)
+            t0 = time.perf_counter()
+            rc1 = lib.amem_mem_pause(0, 0)
+            t1 = time.perf_counter()
+            rc2 = lib.amem_mem_resume(0, 0)
+            t2 = time.perf_counter()
+            assert rc1 == 0 and rc2 == 0, (rc1, rc2)
+            if step >= warmup:
+                pause_s.append(t1 - t0)
+                resume_s.append(t2 - t1)
+                stats.append(H.cycle_stats(lib))
+            elif step == 0:
+                first = (t1 - t0, t2 - t1)
+        return pause_s, resume_s, stats, first
+
+    pause_s, resume_s, stats, first = run_cycles(args.warmup, args.steps)
+
+    # The reference's own structure expressed in HIP calls (one waited-for whole-region copy per
+    # region each way, no scan, no elision), on the same footprint, for comparison only.
+    ref_struct = None
+    if not args.no_reference_structure:
+        path_was = lib.amem_get_option(b"pause_path")
+        assert lib.amem_set_option(b"pause_path", 4) == 0
+        rp, rr, _, _ = run_cycles(1, 5)
+        assert lib.amem_set_option(b"pause_path", path_was) == 0
+        ref_struct = {"value": round(2 * F / statistics.median(a + b for a, b in zip(rp, rr)) / 1e9, 3), "unit": "GB/s",
+                      "p50_pause_s": round(statistics.median(rp), 4), "p50_resume_s": round(statistics.median(rr), 4),
+                      "what": "amem_memPause/amem_memResume loop structure of the reference (amem_nccl.cpp:502-558, "
+                              ":604-630) written with hipMemcpyAsync + sync per region on this GPU; p50 of 5 cycles"}
 
     # correctness gate, outside the clock: bytes, addresses, table
     bad = regs.mismatched_bytes()
@@ -191,6 +212,9 @@ def main():
             "pause_scan_ms", "pause_plan_ms", "pause_copy_ms", "pause_unmap_ms", "resume_map_ms", "resume_copy_ms",
             "k1_ms", "k2_ms", "k3_ms")},
     }
+    if ref_struct:
+        out["reference_structure_on_gpu"] = ref_struct
+        out["speedup_vs_reference_structure"] = round(out["value"] / ref_struct["value"], 3)
     regs.free()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(host_threads)

@@ -264,6 +264,8 @@ int amem_set_enabled(int on);
  *                     2 = 1 when staging memory can be allocated, else 3 (default)
  *                     3 = many short pack launches into pinned host memory, a second host
  *                         thread unmaps each group of regions as soon as its launch is done
+ *                     4 = measurement aid: the reference's own structure in HIP calls (one waited-for
+ *                         whole-region hipMemcpyAsync per region each way, no scan, no elision)
  *   "interleave_bytes" parked bytes per launch of path 3
  *   "dma_min_bytes"   extents at least this long use hipMemcpyAsync in the direct path
  *   "staging_bytes"   size of each of the two device staging buffers

@@ -231,3 +231,19 @@ def test_memstats_output_matches_readme_sample():
     total = [l for l in lines if "in total" in l]
     assert len(total) == 1 and ("total GPU alloc:%d (%d MB)" % (g["total_bytes"], g["total_mb"])) in total[0]
     assert all(l.startswith("AMEM [DEBG] capi.cpp:amem_dump_alloc_stats:") for l in lines)   # the reference's line format
+
+
+def test_headers_compile_and_link_from_c_and_cxx(tmp_path):
+    """include/amem.h is valid C99 for a C compiler, include/amem_nccl.h gives C++ callers the
+    reference's API; both link against the built library and run (registry calls only)."""
+    inc, libdir = os.path.join(ROOT, "include"), os.path.dirname(B.LIB_PATH)
+    env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="1", AMEM_IPC="0", LD_LIBRARY_PATH=libdir + ":" + os.environ.get("LD_LIBRARY_PATH", ""))
+    for compiler, std, src, exe in (("gcc", "-std=c99", "c_caller.c", "c_caller"),
+                                    ("g++", "-std=c++17", "cxx_reference_caller.cpp", "cxx_caller")):
+        out = str(tmp_path / exe)
+        subprocess.run([compiler, std, "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", inc,
+                        os.path.join(ROOT, "tests", "link_check", src), "-o", out, B.LIB_PATH,
+                        "-Wl,-rpath," + libdir], check=True, capture_output=True, text=True)
+        r = subprocess.run([out], env=env, capture_output=True, text=True, timeout=60)
+        assert r.returncode == 0, (r.returncode, r.stdout[-2000:], r.stderr[-2000:])
+        assert "caller ok" in r.stdout

@@ -122,7 +122,8 @@ def test_repeated_cycles_with_writes_between(eng):
 
 @pytest.mark.parametrize("opts", [{"zero_elide": 0}, {"pause_path": 0, "dma_min_bytes": 128 << 10},
                                   {"staging_bytes": 8 << 20}, {"resume_batch_bytes": 1},
-                                  {"staging_bytes": 1 << 20, "resume_batch_bytes": 1 << 40}])
+                                  {"staging_bytes": 1 << 20, "resume_batch_bytes": 1 << 40},
+                                  {"pause_path": 3, "interleave_bytes": 1 << 16}, {"pause_path": 4}])
 def test_option_paths_are_all_bit_exact(eng, opts):
     lib = eng
     for k, v in opts.items():
@@ -137,6 +138,8 @@ def test_option_paths_are_all_bit_exact(eng, opts):
             assert st["parked_bytes"] == fp.total_bytes
         if "dma_min_bytes" in opts:
             assert st["dma_bytes"] > 0 and st["kernel_bytes"] > 0 and st["dma_bytes"] + st["kernel_bytes"] == st["parked_bytes"]
+        if opts.get("pause_path") == 4:
+            assert st["parked_bytes"] == fp.total_bytes and st["k1_launches"] == 0 and st["zero_chunks"] == 0
         if opts.get("staging_bytes") == 1 << 20:
             assert st["kernel_bytes"] > 0                   # regions larger than a staging buffer go direct
         assert lib.amem_mem_resume(0, 0) == 0
