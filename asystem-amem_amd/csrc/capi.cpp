@@ -585,6 +585,7 @@ static OptRef* opt_table(size_t* n) {
       {"resume_batch_bytes", &o.resume_batch_bytes, 1, (int64_t)1 << 40},
       {"peer_timeout_ms", &o.peer_timeout_ms, 0, (int64_t)1 << 40},
       {"peer_loopback", &o.peer_loopback, 0, 1},
+      {"offload_free_tag", &o.offload_free_tag, -1, AMEM_MAX_CALLER - 1},
   };
   *n = sizeof(t) / sizeof(t[0]);
   return t;

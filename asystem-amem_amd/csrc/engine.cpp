@@ -7,6 +7,7 @@
 #include <atomic>
 #include <chrono>
 #include <thread>
+#include <unordered_set>
 
 #include "ipc.h"
 #include "log.h"
@@ -149,13 +150,27 @@ hipError_t Engine::run_scan(const std::vector<ScanSeg>& segs, uint64_t* nchunks_
   return hipSuccess;
 }
 
+// True when [va, va + bytes) lies inside one allocation or mapping known to the runtime.
+// `hint` caches the last range found, since callers pass extents in address order.
+static bool inside_known_memory(uint64_t va, uint64_t bytes, uint64_t hint[2]) {
+  if (bytes == 0) return true;
+  if (va >= hint[0] && va + bytes <= hint[0] + hint[1]) return true;
+  uint64_t base = 0, size = 0;
+  if (!vmm_range_of(va, &base, &size)) return false;
+  hint[0] = base;
+  hint[1] = size;
+  return va >= base && va + bytes <= base + size;
+}
+
 hipError_t Engine::zero_scan(const amem_extent* ext, uint64_t n, uint8_t* flags, amem_chunk_sum* sums,
                              float* ms) {
   hipError_t e = init();
   if (e != hipSuccess) return e;
   std::vector<ScanSeg> segs(n);
+  uint64_t hint[2] = {0, 0};
   for (uint64_t i = 0; i < n; ++i) {
     if ((ext[i].va & 15) || (ext[i].bytes & 15) || ext[i].va == 0) return hipErrorInvalidValue;
+    if (!inside_known_memory(ext[i].va, ext[i].bytes, hint)) return hipErrorInvalidValue;
     segs[i] = {ext[i].va, ext[i].bytes};
   }
   uint64_t total = 0;
@@ -258,9 +273,13 @@ hipError_t Engine::move(bool scatter, const amem_copy_desc* descs, uint64_t n, v
   if (n == 0) return hipSuccess;
   if (!staging || ((uintptr_t)staging & 15)) return hipErrorInvalidValue;
   std::vector<CopyDesc> v(n);
+  uint64_t hint[2] = {0, 0};
+  if (!inside_known_memory((uint64_t)(uintptr_t)staging, staging_bytes, hint)) return hipErrorInvalidValue;
+  hint[0] = hint[1] = 0;
   for (uint64_t i = 0; i < n; ++i) {
     const amem_copy_desc& d = descs[i];
     if (d.va == 0 || (d.va & 15) || (d.bytes & 15)) return hipErrorInvalidValue;
+    if (!inside_known_memory(d.va, d.bytes, hint)) return hipErrorInvalidValue;
     if (d.off == kDescZero) {
       if (!scatter) return hipErrorInvalidValue;
     } else if ((d.off & 15) || d.off > staging_bytes || d.bytes > staging_bytes - d.off) {
@@ -606,7 +625,7 @@ int Engine::pause(Ctx& c) {
   LOGGER(INFO, "memPause: groupID:%d pid:%d GPU:%d memUsed: %ld MB before paused", amem_groupID_value(),
          getpid(), dev_, (long)((total - free_sz) >> 20));
 
-  std::vector<Region*> locals;
+  std::vector<Region*> locals, invalid;
   std::vector<std::pair<uint64_t, Region*>> imported;
   parked_.clear();
   gather_descs_.clear();
@@ -616,10 +635,24 @@ int Engine::pause(Ctx& c) {
     if (r.state != AMEM_STATE_ALLOC) continue;
     if (from_peer(r.type)) imported.push_back({kv.first, &r});
     else {
+      // A kernel must never be pointed at memory that is not there: a region whose VA is not
+      // (or no longer) mapped over its whole registered size is reported and not read.
+      uint64_t base = 0, msize = 0;
+      if ((kv.first & 15) || (r.allocSz & 15) || r.allocSz == 0 || !vmm_range_of(kv.first, &base, &msize) ||
+          base != kv.first || msize < r.allocSz) {
+        LOGGER(ERROR, "memPause: groupID:%d pid:%d dptr:%llx allocSz:%ld is not a mapped, 16-byte aligned range "
+               "(mapping base:%llx size:%ld); its bytes are not saved", amem_groupID_value(), getpid(),
+               (unsigned long long)kv.first, (long)r.allocSz, (unsigned long long)base, (long)msize);
+        if (rc == 0) rc = (int)hipErrorInvalidValue;
+        invalid.push_back(&r);
+        continue;
+      }
       locals.push_back(&r);
       segs_.push_back({kv.first, (uint64_t)r.allocSz});
     }
   }
+  const int rc_validation = rc;
+  rc = 0;  // the valid regions are still paused; the validation error is returned at the end
 
   // Imported mappings go first (reference step 2, amem_nccl.cpp:517-526): no data to save,
   // and the owner's release only frees memory once importers have let go.
@@ -678,7 +711,13 @@ int Engine::pause(Ctx& c) {
     p.nchunks = chunks_of(p.size);
     p.parked_off = cursor;
     p.desc_begin = (uint32_t)gather_descs_.size();
-    emit_runs(flags + chunk0, p.va, p.size, elide, &cursor, slab_bytes, &gather_descs_, nullptr, &zero_chunks);
+    // Regions registered under the offload-free caller tag are scratch: released without being
+    // copied and handed back zero-filled (README.md:224 of the reference describes the intent;
+    // its own comparison against the tag never takes effect, amem_nccl.cpp:40, :503, :620).
+    p.skip = !ref_mode_ && options().offload_free_tag >= 0 && (int64_t)locals[i]->tags == options().offload_free_tag;
+    if (p.skip) std::fill(parked_flags_.begin() + chunk0, parked_flags_.begin() + chunk0 + p.nchunks, (uint8_t)1);
+    emit_runs(flags + chunk0, p.va, p.size, elide || p.skip, &cursor, slab_bytes, &gather_descs_, nullptr,
+              p.skip ? nullptr : &zero_chunks);
     p.desc_end = (uint32_t)gather_descs_.size();
     p.parked_bytes = cursor - p.parked_off;
     chunk0 += p.nchunks;
@@ -739,7 +778,7 @@ int Engine::pause(Ctx& c) {
          amem_groupID_value(), getpid(), dev_, (long)c.pauseCnt, (long)((total - free_sz) >> 20),
          (long)(stats_.footprint_bytes >> 20), (long)stats_.pause_ms, c.offloadCnt, c.releaseLocalCnt,
          c.releaseShadowCnt);
-  return rc;
+  return rc ? rc : rc_validation;
 }
 
 void Engine::forget(uint64_t va) {
@@ -784,7 +823,7 @@ int Engine::resume(Ctx& c) {
     Item im = {&r, p.va, (uint32_t)scatter.size(), 0, p.size};
     uint64_t cursor = p.parked_off;
     std::vector<CopyDesc> zeros;
-    emit_runs(flags + p.first_chunk, p.va, p.size, elide, &cursor, slab_bytes, &scatter, &zeros, nullptr);
+    emit_runs(flags + p.first_chunk, p.va, p.size, elide || p.skip, &cursor, slab_bytes, &scatter, &zeros, nullptr);
     scatter.insert(scatter.end(), zeros.begin(), zeros.end());
     im.d1 = (uint32_t)scatter.size();
     items.push_back(im);
@@ -792,12 +831,12 @@ int Engine::resume(Ctx& c) {
     verify_first_chunk.push_back(p.first_chunk);
   }
   // Local holes that were never saved come back as zeros.
+  std::unordered_set<uint64_t> item_vas;
+  for (const Item& im : items) item_vas.insert(im.va);
   for (auto& kv : table) {
     Region& r = kv.second;
     if (r.state != AMEM_STATE_HOLE || from_peer(r.type)) continue;
-    bool known = false;
-    for (const Item& im : items) if (im.va == kv.first) { known = true; break; }
-    if (known) continue;
+    if (item_vas.count(kv.first)) continue;
     Item im = {&r, kv.first, (uint32_t)scatter.size(), 0, (uint64_t)r.allocSz};
     scatter.push_back({kv.first, kDescZero, (uint64_t)r.allocSz & ~(uint64_t)15});
     im.d1 = (uint32_t)scatter.size();

@@ -28,6 +28,7 @@ struct Options {
   int64_t hbm_wgs = 65536;                // workgroup cap of device-only kernels
   int64_t resume_batch_bytes = 64ll << 20;
   int64_t peer_timeout_ms = 60000;
+  int64_t offload_free_tag = -1;          // caller tag whose regions are released without being copied
   int64_t peer_loopback = 0;              // let a process register with / update its own service (tests)
 };
 Options& options();
@@ -54,6 +55,7 @@ struct ParkedRegion {
   uint64_t parked_off;    // logical pool offset of the first parked byte
   uint64_t parked_bytes;
   uint32_t desc_begin, desc_end;  // range in gather_descs_
+  bool skip;              // registered under the offload-free tag: nothing parked, zeros restored
 };
 
 class Engine {

@@ -75,6 +75,18 @@ uint64_t vmm_handle_of(uint64_t va) {
   return handle_bits(h);
 }
 
+bool vmm_range_of(uint64_t addr, uint64_t* base, uint64_t* size) {
+  hipDeviceptr_t b = nullptr;
+  size_t s = 0;
+  if (hipMemGetAddressRange(&b, &s, (hipDeviceptr_t)(uintptr_t)addr) != hipSuccess || s == 0) {
+    (void)hipGetLastError();
+    return false;
+  }
+  *base = (uint64_t)(uintptr_t)b;
+  *size = s;
+  return true;
+}
+
 // Size of the mapping that starts at `va` (cuMemGetAddressRange in amem_cuMemReleaseHandle,
 // amem_nccl.h:150), or `fallback` when the runtime cannot tell.
 static size_t mapped_size(uint64_t va, size_t fallback) {

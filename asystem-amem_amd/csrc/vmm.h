@@ -41,6 +41,8 @@ hipError_t vmm_export_fd(uint64_t handle, int* fd);
 // when `close_fd`.
 hipError_t vmm_import_map(int dev, uint64_t va, size_t size, int fd, bool close_fd,
                           uint64_t* new_handle);
+// Allocation or mapping that contains `addr`: its base and size. False when the runtime knows none.
+bool vmm_range_of(uint64_t addr, uint64_t* base, uint64_t* size);
 // Handle currently mapped at `va`, 0 if none. Takes no reference.
 uint64_t vmm_handle_of(uint64_t va);
 // Device that owns the physical memory behind `handle`, -1 if unknown.

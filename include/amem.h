@@ -272,6 +272,11 @@ int amem_set_enabled(int on);
  *   "slab_bytes"      size of one pinned host slab (power of two)
  *   "link_wgs"        workgroups of a kernel that reads or writes host memory
  *   "peer_timeout_ms" how long resume waits for owners before failing (0 = forever)
+ *   "offload_free_tag" caller tag (0-15, -1 = none) whose regions hold scratch data: pause releases
+ *                     them without copying and resume hands them back zero-filled. This is what
+ *                     AMEM_NCCL_OFFLOAD_FREE_TAG is documented to do in the reference, where the
+ *                     variable is parsed but never takes effect (amem_nccl.cpp:40, :503, :620);
+ *                     the environment variable stays ineffective here too, only this option acts
  *   "peer_loopback"   0/1   treat this process's own slot like any other peer: registration and
  *                     re-export go through the socket service of the same process (default 0:
  *                     a process never registers with itself, gmm_client_impl.cpp:482-484, :512-514) */

@@ -259,3 +259,63 @@ def test_full_size_headline_footprint_one_cycle(eng):
     assert H.compare_tables(before, regs.table()) == []
     assert st["pause_ms"] + st["resume_ms"] < 1000.0          # the headline target: under one second
     regs.free()
+
+
+def test_offload_free_tag_releases_without_copy(eng):
+    """Regions registered under the offload-free caller tag are scratch: not copied, handed back
+    zero-filled; everything else is untouched (the reference documents this for
+    AMEM_NCCL_OFFLOAD_FREE_TAG, README.md:224, but never applies it)."""
+    lib = eng
+    assert lib.amem_set_option(b"offload_free_tag", B.CALLER_PROXY) == 0
+    try:
+        rng = np.random.default_rng(21)
+        items = []
+        for k, caller in enumerate([B.CALLER_P2P, B.CALLER_PROXY, B.CALLER_P2P]):
+            va, h, asz = C.c_uint64(), C.c_uint64(), C.c_uint64()
+            assert lib.amem_vmm_alloc(4 * MiB, 0, C.byref(va), C.byref(h), C.byref(asz)) == 0
+            data = rng.integers(1, 256, 4 * MiB, dtype=np.uint8)
+            lib.amem_copy_to_device(va.value, data.ctypes.data, data.nbytes)
+            assert lib.amem_add_alloc_info(va.value, asz.value, 0, 0, h.value, -1, 0, None, caller) == 0
+            items.append((va.value, asz.value, data, caller))
+        assert lib.amem_mem_pause(0, 0) == 0
+        st = H.cycle_stats(lib)
+        assert st["parked_bytes"] == 8 * MiB and st["footprint_bytes"] == 12 * MiB and st["zero_chunks"] == 0
+        assert lib.amem_mem_resume(0, 0) == 0
+        for va, asz, data, caller in items:
+            out = np.empty(4 * MiB, dtype=np.uint8)
+            lib.amem_copy_from_device(out.ctypes.data, va, out.nbytes)
+            assert np.array_equal(out, data) if caller != B.CALLER_PROXY else not out.any()
+            lib.amem_del_alloc_info(va, 0, 0)
+            lib.amem_vmm_free(va, asz, 0)
+    finally:
+        lib.amem_mem_resume(0, 0)
+        assert lib.amem_set_option(b"offload_free_tag", -1) == 0
+
+
+def test_stale_registration_is_reported_not_read(eng):
+    """A region registered with more bytes than are mapped must not be handed to a kernel: pause
+    reports it, saves the others, and the GPU takes no fault."""
+    lib = eng
+    good, bad = [C.c_uint64() for _ in range(3)], [C.c_uint64() for _ in range(3)]
+    assert lib.amem_vmm_alloc(4 * MiB, 0, C.byref(good[0]), C.byref(good[1]), C.byref(good[2])) == 0
+    assert lib.amem_vmm_alloc(2 * MiB, 0, C.byref(bad[0]), C.byref(bad[1]), C.byref(bad[2])) == 0
+    data = np.random.default_rng(4).integers(1, 256, 4 * MiB, dtype=np.uint8)
+    lib.amem_copy_to_device(good[0].value, data.ctypes.data, data.nbytes)
+    assert lib.amem_add_alloc_info(good[0].value, good[2].value, 0, 0, good[1].value, -1, 0, None, 1) == 0
+    assert lib.amem_add_alloc_info(bad[0].value, 64 * MiB, 0, 0, bad[1].value, -1, 0, None, 1) == 0   # 62 MiB too many
+    assert lib.amem_mem_pause(0, 0) != 0
+    st = H.cycle_stats(lib)
+    assert st["local_regions"] == 1 and st["footprint_bytes"] == 4 * MiB
+    assert lib.amem_check_paused(0) == 1
+    lib.amem_del_alloc_info(bad[0].value, 0, 0)                        # the caller cleans its stale entry up
+    assert lib.amem_mem_resume(0, 0) == 0
+    out = np.empty(4 * MiB, dtype=np.uint8)
+    lib.amem_copy_from_device(out.ctypes.data, good[0].value, out.nbytes)
+    assert np.array_equal(out, data)
+    lib.amem_del_alloc_info(good[0].value, 0, 0)
+    lib.amem_vmm_free(good[0].value, good[2].value, 0)
+    lib.amem_vmm_free(bad[0].value, bad[2].value, 0)                   # pause unmapped it; the reservation is freed here
+    # the kernels' own entry points refuse ranges the runtime does not know
+    ext = (B.Extent * 1)(B.Extent(0x7e0000000000, 65536))
+    one = (C.c_uint8 * 1)()
+    assert lib.amem_zero_scan(ext, 1, one, None, None) != 0
