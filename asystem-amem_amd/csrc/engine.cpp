@@ -307,7 +307,7 @@ hipError_t Engine::move(bool scatter, const amem_copy_desc* descs, uint64_t n, v
   (void)CHECK_HIP(hipEventRecord(e0, kstream_));
   e = CHECK_HIP(launch_move(scatter, (const CopyDesc*)d_descs_.p, (const uint64_t*)d_tiles_.p,
                             (uint32_t)n, 0, ntiles, st, 0,
-                            (uint32_t)(host_side ? options().link_wgs : options().hbm_wgs), kstream_));
+                            (uint32_t)(host_side ? options().link_wgs : options().hbm_wgs), 8, kstream_));
   if (e != hipSuccess) return e;
   (void)CHECK_HIP(hipEventRecord(e1, kstream_));
   e = CHECK_HIP(hipStreamSynchronize(kstream_));
@@ -400,7 +400,7 @@ hipError_t Engine::pause_copy_direct(Ctx& c, std::vector<Region*>& regs) {
   hipEvent_t e0 = event_at(4), e1 = event_at(5);
   (void)CHECK_HIP(hipEventRecord(e0, kstream_));
   e = CHECK_HIP(launch_move(false, (const CopyDesc*)d_descs_.p, (const uint64_t*)d_tiles_.p,
-                            (uint32_t)kdescs.size(), 0, ntiles, st, 0, (uint32_t)options().link_wgs, kstream_));
+                            (uint32_t)kdescs.size(), 0, ntiles, st, 0, (uint32_t)options().link_wgs, 8, kstream_));
   if (e != hipSuccess) return e;
   (void)CHECK_HIP(hipEventRecord(e1, kstream_));
   if (ntiles) stats_.k2_launches++;
@@ -468,7 +468,7 @@ hipError_t Engine::pause_copy_interleaved(Ctx& c, std::vector<Region*>& regs) {
     if (G.d1 > G.d0 && tp[G.d1] > tp[G.d0]) {
       e = CHECK_HIP(launch_move(false, (const CopyDesc*)d_descs_.p + G.d0, (const uint64_t*)d_tiles_.p + G.d0,
                                 G.d1 - G.d0, tp[G.d0], tp[G.d1] - tp[G.d0], pool_tab, 0,
-                                (uint32_t)options().link_wgs, kstream_));
+                                (uint32_t)options().pause_wgs, (uint32_t)options().pause_xcds, kstream_));
       if (e != hipSuccess) break;
       stats_.k2_launches++;
       stats_.kernel_bytes += G.bytes;
@@ -548,7 +548,7 @@ hipError_t Engine::pause_copy_staged(Ctx& c, std::vector<Region*>& regs, bool* u
         (void)CHECK_HIP(hipEventRecord(s0, kstream_));
         e = CHECK_HIP(launch_move(false, (const CopyDesc*)d_descs_.p + d0, (const uint64_t*)d_tiles_.p + d0,
                                   d1 - d0, tp[d0], tp[d1] - tp[d0], pool_tab, 0,
-                                  (uint32_t)options().link_wgs, kstream_));
+                                  (uint32_t)options().link_wgs, 8, kstream_));
         if (e != hipSuccess) return e;
         (void)CHECK_HIP(hipEventRecord(s1, kstream_));
         e = CHECK_HIP(hipEventSynchronize(s1));
@@ -564,7 +564,7 @@ hipError_t Engine::pause_copy_staged(Ctx& c, std::vector<Region*>& regs, bool* u
         (void)CHECK_HIP(hipEventRecord(s0, kstream_));
         e = CHECK_HIP(launch_move(false, (const CopyDesc*)d_descs_.p + d0, (const uint64_t*)d_tiles_.p + d0,
                                   d1 - d0, tp[d0], tp[d1] - tp[d0], stg, base,
-                                  (uint32_t)options().hbm_wgs, kstream_));
+                                  (uint32_t)options().hbm_wgs, 8, kstream_));
         if (e != hipSuccess) return e;
         (void)CHECK_HIP(hipEventRecord(s1, kstream_));
         e = CHECK_HIP(hipEventSynchronize(s1));
@@ -741,11 +741,11 @@ int Engine::pause(Ctx& c) {
     if (ref_mode_) {
       note(pause_copy_reference(c, locals));
       staged = true;
-    } else if (path == 3 && !locals.empty()) {
+    } else if ((path == 3 || path == 2) && !locals.empty()) {
       note(upload_slab_table());
       note(pause_copy_interleaved(c, locals));
       staged = true;
-    } else if (path != 0 && !locals.empty()) {
+    } else if (path == 1 && !locals.empty()) {
       note(pause_copy_staged(c, locals, &staged));
     }
     if (!staged && rc == 0) {
@@ -906,7 +906,7 @@ int Engine::resume(Ctx& c) {
       (void)CHECK_HIP(hipEventRecord(s0, kstream_));
       note(CHECK_HIP(launch_move(true, (const CopyDesc*)d_descs_.p + d0, (const uint64_t*)d_tiles_.p + d0,
                                  d1 - d0, tp[d0], tp[d1] - tp[d0], pool_tab, 0,
-                                 (uint32_t)options().link_wgs, kstream_)));
+                                 (uint32_t)options().link_wgs, 8, kstream_)));
       (void)CHECK_HIP(hipEventRecord(s1, kstream_));
       timed.push_back({s0, s1});
       stats_.k3_launches++;

@@ -43,7 +43,7 @@ hipError_t launch_scan(const ScanSeg* d_segs, const uint64_t* d_chunk_prefix, ui
 
 hipError_t launch_move(bool scatter, const CopyDesc* d_descs, const uint64_t* d_tile_prefix,
                        uint32_t ndescs, uint64_t first_tile, uint64_t ntiles,
-                       const SlabTable& slabs, uint64_t off_base, uint32_t max_blocks,
+                       const SlabTable& slabs, uint64_t off_base, uint32_t max_blocks, uint32_t xcds,
                        hipStream_t stream);
 
 hipError_t launch_calib_copy(const void* d_src, void* d_dst, uint64_t bytes, hipStream_t stream);

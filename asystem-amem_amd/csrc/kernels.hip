@@ -23,6 +23,7 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 static constexpr int kWave = 64;
 static constexpr int kBlock = 256;
 static constexpr int kWavesPerBlock = kBlock / kWave;
+static constexpr uint32_t kXcds = 8;  // accelerator complex dies of the MI355X
 
 // Largest index i in [0, n) with prefix[i] <= x, for a non-decreasing prefix[0..n] with
 // prefix[0] <= x < prefix[n].
@@ -127,14 +128,23 @@ __device__ __forceinline__ uint8_t* slab_addr(const SlabTable& t, uint64_t off) 
 // of a long descriptor list can be packed into a buffer that starts at that offset.
 //   MODE 0  gather : staging[off + o] = device[va + o]
 //   MODE 1  scatter: device[va + o] = staging[off + o], or zeros when off == kDescZero
+// `xcds` confines the work to the first `xcds` of the chip's 8 XCDs: workgroups are dealt to
+// XCDs round-robin by workgroup id, so a workgroup whose id modulo 8 is >= xcds retires at
+// once and the others renumber themselves densely. A host-side hipMemUnmap issued while a
+// kernel runs has to wait for a TLB shoot-down on every XCD that has waves in flight
+// (measured: 0.43 ms with one XCD busy, 0.55 ms with two, 2.2 ms with all eight), while one
+// XCD alone already drives the host link at 52 of its 57 GB/s.
 template <int MODE>
 __global__ __launch_bounds__(kBlock) void move_tiles(const CopyDesc* __restrict__ descs,
                                                      const uint64_t* __restrict__ tile_prefix,
                                                      uint32_t ndescs, uint64_t first_tile,
                                                      uint64_t ntiles, SlabTable slabs,
-                                                     uint64_t off_base) {
+                                                     uint64_t off_base, uint32_t xcds) {
   const uint32_t tid = threadIdx.x;
-  for (uint64_t tt = blockIdx.x; tt < ntiles; tt += gridDim.x) {
+  if ((blockIdx.x & (kXcds - 1)) >= xcds) return;
+  const uint64_t wg = (uint64_t)(blockIdx.x / kXcds) * xcds + (blockIdx.x & (kXcds - 1));
+  const uint64_t nwg = (uint64_t)(gridDim.x / kXcds) * xcds;
+  for (uint64_t tt = wg; tt < ntiles; tt += nwg) {
     const uint64_t t = first_tile + tt;
     const uint32_t d = find_segment(tile_prefix, ndescs, t);
     const uint64_t o = (t - tile_prefix[d]) * kTileBytes;
@@ -200,17 +210,21 @@ hipError_t launch_scan(const ScanSeg* d_segs, const uint64_t* d_chunk_prefix, ui
 
 hipError_t launch_move(bool scatter, const CopyDesc* d_descs, const uint64_t* d_tile_prefix,
                        uint32_t ndescs, uint64_t first_tile, uint64_t ntiles,
-                       const SlabTable& slabs, uint64_t off_base, uint32_t max_blocks,
+                       const SlabTable& slabs, uint64_t off_base, uint32_t max_blocks, uint32_t xcds,
                        hipStream_t stream) {
   if (ntiles == 0 || ndescs == 0) return hipSuccess;
-  const uint32_t grid = clamp_grid(ntiles, max_blocks);
+  if (xcds < 1 || xcds > kXcds) xcds = kXcds;
+  // the grid is a multiple of 8 so that every XCD is dealt the same number of workgroups;
+  // `max_blocks` counts the workgroups that actually work
+  const uint32_t per_xcd = (clamp_grid(ntiles, max_blocks) + xcds - 1) / xcds;
+  const uint32_t grid = per_xcd * kXcds;
   (void)hipGetLastError();
   if (scatter)
     hipLaunchKernelGGL(move_tiles<1>, dim3(grid), dim3(kBlock), 0, stream, d_descs, d_tile_prefix,
-                       ndescs, first_tile, ntiles, slabs, off_base);
+                       ndescs, first_tile, ntiles, slabs, off_base, xcds);
   else
     hipLaunchKernelGGL(move_tiles<0>, dim3(grid), dim3(kBlock), 0, stream, d_descs, d_tile_prefix,
-                       ndescs, first_tile, ntiles, slabs, off_base);
+                       ndescs, first_tile, ntiles, slabs, off_base, xcds);
   return hipGetLastError();
 }
 

@@ -259,14 +259,18 @@ int amem_set_enabled(int on);
 /* Tunables. Unknown name or bad value returns 1. Names:
  *   "zero_elide"      0/1   skip all-zero 64 KiB chunks (default 1)
  *   "verify"          0/1   re-scan after resume and compare checksums (default 0)
- *   "pause_path"      0 = one pack kernel writes pinned host memory, then regions are unmapped
- *                     1 = pack into device staging, large hipMemcpyAsync, unmap during the transfer
- *                     2 = 1 when staging memory can be allocated, else 3 (default)
- *                     3 = many short pack launches into pinned host memory, a second host
+ *   "pause_path"      how pause moves bytes and overlaps the unmaps:
+ *                     0 = one pack kernel writes pinned host memory, then regions are unmapped
+ *                     1 = pack into device staging, large hipMemcpyAsync, unmap meanwhile
+ *                     3 = many short pack launches into pinned host memory, confined to
+ *                         "pause_xcds" XCDs and "pause_wgs" workgroups, while a second host
  *                         thread unmaps each group of regions as soon as its launch is done
+ *                     2 = the default, currently 3
  *                     4 = measurement aid: the reference's own structure in HIP calls (one waited-for
  *                         whole-region hipMemcpyAsync per region each way, no scan, no elision)
- *   "interleave_bytes" parked bytes per launch of path 3
+ *   "interleave_bytes" parked bytes per launch of path 3 (default 4 MiB)
+ *   "pause_wgs"       workgroups of path 3's pack kernel (default 4)
+ *   "pause_xcds"      XCDs those workgroups are confined to (default 1, at most 8)
  *   "dma_min_bytes"   extents at least this long use hipMemcpyAsync in the direct path
  *   "staging_bytes"   size of each of the two device staging buffers
  *   "slab_bytes"      size of one pinned host slab (power of two)
