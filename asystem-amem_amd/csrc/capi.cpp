@@ -620,16 +620,13 @@ int64_t amem_get_option(const char* name) {
 
 uint64_t amem_pool_trim(void) {
   Ctx* c = ctx_or_null();
-  if (c) {
+  if (!c) return 0;
+  std::lock_guard<std::mutex> ls(c->structure);  // not while a pause or resume is running
+  {
     std::lock_guard<std::mutex> lf(c->fields);
-    if (c->paused) return 0;
+    if (c->paused) return 0;  // the pool holds the parked bytes
   }
-  uint64_t freed = 0;
-  for (int d = 0; d < AMEM_MAX_DEVS; ++d) {
-    // engines exist only for devices that were paused at least once
-    if (c && c->engine && d == current_device()) freed += c->engine->trim_pool();
-  }
-  return freed;
+  return c->engine ? c->engine->trim_pool() : 0;
 }
 
 int amem_shutdown(void) {

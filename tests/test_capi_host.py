@@ -132,7 +132,7 @@ def test_region_order_and_find(fresh):
 
 
 def test_registry_latency_with_100k_entries(fresh):
-    """The registry side of BASELINE config 4: 100,000 entries inserted, looked up and deleted.
+    """The registry side of benchmark configuration 4: 100,000 entries inserted, looked up and deleted.
     The bound is loose (shared CI cores); the measured figure is printed."""
     import time
     lib = fresh

@@ -58,7 +58,7 @@ def same_as_oracle(lib, orc, vas, twin):
 
 @pytest.mark.parametrize("path", [0, 1, 3])
 def test_config2_cycle_bit_exact_same_va_same_table(eng, fresh_orc, path):
-    """BASELINE config 2: 256 regions (128x4 + 96x2 + 32x16 MiB), half of the 64 KiB chunks zero."""
+    """benchmark configuration 2: 256 regions (128x4 + 96x2 + 32x16 MiB), half of the 64 KiB chunks zero."""
     lib, orc = eng, fresh_orc
     assert lib.amem_set_option(b"pause_path", path) == 0
     fp = Footprint(2, 1, threads=16)
@@ -96,7 +96,7 @@ def test_config2_cycle_bit_exact_same_va_same_table(eng, fresh_orc, path):
 
 
 def test_repeated_cycles_with_writes_between(eng):
-    """BASELINE config 3 at 1 GiB: repeated cycles, 1 % of chunks rewritten in between,
+    """benchmark configuration 3 at 1 GiB: repeated cycles, 1 % of chunks rewritten in between,
     including zero -> non-zero and non-zero -> zero flips."""
     lib = eng
     fp = Footprint(3, 2, byte_budget=1 << 30, threads=16)

@@ -170,7 +170,7 @@ def test_pack_unpack_match_oracle(gpu, orc, host_side):
 
 @pytest.mark.parametrize("count", [2000, 100000])
 def test_fragmented_descriptor_list_round_trip(gpu, orc, count):
-    """BASELINE config 4 (100,000 sub-allocations of 4-64 KiB bump-packed into 2 MiB granules, seed 3;
+    """benchmark configuration 4 (100,000 sub-allocations of 4-64 KiB bump-packed into 2 MiB granules, seed 3;
     also at 1/50 scale): gathered into contiguous staging and scattered back into fresh memory."""
     fp = Footprint(4, 3, max_regions=count, threads=16)
     granule = 2 * MiB

@@ -1,4 +1,4 @@
-"""Several processes sharing the one GPU (BASELINE config 5 at reduced size): every process
+"""Several processes sharing the one GPU (benchmark configuration 5 at reduced size): every process
 owns regions, exports them as POSIX fds, imports all peers' regions; coordinated pause (importers
 let go first, owners' release then frees the memory) and resume (owners re-create and re-export,
 importers remap at their original VA). Reference: amem_nccl.cpp:517-526, :633-662, R10 of the

@@ -37,7 +37,7 @@ def make_local(orc, ctx, fp, caller=1):
 
 
 def test_config1_cycle_identity_table_and_release(fresh_orc):
-    """BASELINE config 1 at a quarter of its size (16 of the 64 regions): host-memcpy pause to
+    """benchmark configuration 1 at a quarter of its size (16 of the 64 regions): host-memcpy pause to
     a host buffer then restore; byte compare plus region-table compare."""
     orc = fresh_orc
     fp = Footprint(1, 0, max_regions=16)
