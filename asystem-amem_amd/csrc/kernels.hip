@@ -24,6 +24,7 @@ static constexpr int kWave = 64;
 static constexpr int kBlock = 256;
 static constexpr int kWavesPerBlock = kBlock / kWave;
 static constexpr uint32_t kXcds = 8;  // accelerator complex dies of the MI355X
+static constexpr int kRounds = (int)(kTileBytes / (kBlock * 16));  // 16-byte loads a lane keeps in flight per tile
 
 // Largest index i in [0, n) with prefix[i] <= x, for a non-decreasing prefix[0..n] with
 // prefix[0] <= x < prefix[n].
@@ -123,8 +124,8 @@ __device__ __forceinline__ uint8_t* slab_addr(const SlabTable& t, uint64_t off) 
 // Tile mover. Descriptor d covers tiles [tile_prefix[d], tile_prefix[d+1]) of kTileBytes
 // each (the last tile of a descriptor may be shorter); a launch handles the `ndescs`
 // descriptors whose tiles are [first_tile, first_tile + ntiles). A workgroup takes tiles
-// grid-stride; within a tile, 256 lanes x 16 B = 4 KiB per round, four rounds loaded
-// before any store. `off_base` is subtracted from every descriptor offset, so a sub-range
+// grid-stride; within a tile, 256 lanes x 16 B = 4 KiB per round, all rounds of the tile
+// loaded before any store. `off_base` is subtracted from every descriptor offset, so a sub-range
 // of a long descriptor list can be packed into a buffer that starts at that offset.
 //   MODE 0  gather : staging[off + o] = device[va + o]
 //   MODE 1  scatter: device[va + o] = staging[off + o], or zeros when off == kDescZero
@@ -162,15 +163,12 @@ __global__ __launch_bounds__(kBlock) void move_tiles(const CopyDesc* __restrict_
     const u32x4* __restrict__ src = (MODE == 0) ? dev : stg;
     u32x4* __restrict__ dst = (MODE == 0) ? stg : dev;
     uint32_t i = tid;
-    for (; i + 3 * kBlock < nvec; i += 4 * kBlock) {
-      u32x4 a = __builtin_nontemporal_load(src + i);
-      u32x4 b = __builtin_nontemporal_load(src + i + kBlock);
-      u32x4 c = __builtin_nontemporal_load(src + i + 2 * kBlock);
-      u32x4 e = __builtin_nontemporal_load(src + i + 3 * kBlock);
-      __builtin_nontemporal_store(a, dst + i);
-      __builtin_nontemporal_store(b, dst + i + kBlock);
-      __builtin_nontemporal_store(c, dst + i + 2 * kBlock);
-      __builtin_nontemporal_store(e, dst + i + 3 * kBlock);
+    for (; i + (kRounds - 1) * kBlock < nvec; i += kRounds * kBlock) {
+      u32x4 v[kRounds];
+#pragma unroll
+      for (int r = 0; r < kRounds; ++r) v[r] = __builtin_nontemporal_load(src + i + r * kBlock);
+#pragma unroll
+      for (int r = 0; r < kRounds; ++r) __builtin_nontemporal_store(v[r], dst + i + r * kBlock);
     }
     for (; i < nvec; i += kBlock) {
       u32x4 a = __builtin_nontemporal_load(src + i);

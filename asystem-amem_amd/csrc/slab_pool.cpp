@@ -16,6 +16,8 @@ SlabPool::~SlabPool() { trim(); }
 hipError_t SlabPool::ensure(uint64_t bytes) {
   while (capacity() < bytes) {
     void* p = nullptr;
+    // Default flags: coherent / non-coherent / portable / NUMA-user variants measured the same
+    // for both the copy engine and kernels that read or write the slab.
     hipError_t e = CHECK_HIP(hipHostMalloc(&p, slab_bytes_, hipHostMallocDefault));
     if (e != hipSuccess) return e;
     slabs_.push_back((uint8_t*)p);
