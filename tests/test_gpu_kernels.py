@@ -131,10 +131,16 @@ def test_pack_unpack_match_oracle(gpu, orc, host_side):
         pieces.append((a, off, n))
         off += n + 32            # leave gaps in staging: they must stay untouched
     total = off
-    import torch
     if host_side:
-        stage_t = torch.full((total,), 0xCC, dtype=torch.uint8).pin_memory()
-        stage_ptr = stage_t.data_ptr()
+        # pinned host memory straight from the HIP runtime the library is linked against
+        hip = C.CDLL("libamdhip64.so")
+        hip.hipHostMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t, C.c_uint]
+        hip.hipHostFree.argtypes = [C.c_void_p]
+        pinned = C.c_void_p()
+        assert hip.hipHostMalloc(C.byref(pinned), total, 0) == 0
+        stage_ptr = pinned.value
+        stage_np = np.frombuffer((C.c_uint8 * total).from_address(stage_ptr), dtype=np.uint8)
+        stage_np[:] = 0xCC
     else:
         stage = DevBuf(gpu, total)
         stage.put(np.full(stage.alloc, 0xCC, dtype=np.uint8))
@@ -143,7 +149,7 @@ def test_pack_unpack_match_oracle(gpu, orc, host_side):
     rc = gpu.amem_gather_pack(_descs([(src.va + a, o, n) for a, o, n in pieces]), len(pieces), stage_ptr, total,
                               host_side, C.byref(ms))
     assert rc == 0
-    got = stage_t.numpy().copy() if host_side else stage.get(total)
+    got = stage_np.copy() if host_side else stage.get(total)
     want = np.full(total, 0xCC, dtype=np.uint8)
     od = (O.CopyDesc * len(pieces))(*[O.CopyDesc(data.ctypes.data + a, o, n) for a, o, n in pieces])
     orc.oracle_gather_pack(od, len(pieces), want.ctypes.data)
@@ -164,7 +170,10 @@ def test_pack_unpack_match_oracle(gpu, orc, host_side):
     assert gpu.amem_gather_pack(_descs([(src.va, B.DESC_ZERO, 32)]), 1, stage_ptr, total, host_side, None) != 0
     assert gpu.amem_gather_pack(_descs([]), 0, stage_ptr, total, host_side, None) == 0
     src.free(); dst.free()
-    if not host_side:
+    if host_side:
+        del stage_np
+        assert hip.hipHostFree(pinned) == 0
+    else:
         stage.free()
 
 
