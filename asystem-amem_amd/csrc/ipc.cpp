@@ -227,12 +227,14 @@ int rpc(int slot, const WireReq& req, int fd) {
   int s = connect_if_not(slot);
   if (s < 0) return 1;
   int32_t ret = 1;
-  if (send_msg(s, &req, sizeof(req), fd) > 0) {
-    if (recv_msg(s, &ret, sizeof(ret), nullptr) != (ssize_t)sizeof(ret)) ret = 1;
-  }
-  if (ret != 0) {
-    // a broken connection is not reused
-    if (errno == EPIPE || errno == ECONNRESET || errno == EAGAIN) { close(s); g_svc.conn[slot] = -1; }
+  const bool sent = send_msg(s, &req, sizeof(req), fd) == (ssize_t)sizeof(req);
+  const bool answered = sent && recv_msg(s, &ret, sizeof(ret), nullptr) == (ssize_t)sizeof(ret);
+  if (!answered) {
+    // peer gone, or no answer within the timeout: drop the connection so that the next
+    // request reconnects instead of reading a stale reply
+    close(s);
+    g_svc.conn[slot] = -1;
+    return 1;
   }
   return ret;
 }
