@@ -11,6 +11,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIBNAME = "libamem_nccl.so.1"
+HOOK_NAME = "libamem_rccl_hook.so"
 HIP_SOURCES = ["kernels.hip"]
 CXX_SOURCES = ["capi.cpp", "engine.cpp", "ipc.cpp", "log.cpp", "slab_pool.cpp", "vmm.cpp"]
 # The packed-fp32 target feature is switched off for all device code of this project.
@@ -38,6 +39,14 @@ def build(verbose=True):
         objs.append(obj)
     out = lib_path()
     cmd = [hipcc, "-shared", "-fPIC", "-Wl,-soname," + LIBNAME, "--offload-arch=gfx950", "-o", out] + objs + ["-lpthread"]
+    _run(cmd, verbose)
+    # the allocator hook for an unpatched RCCL: host code only, placed in front of the HIP runtime
+    hook = os.path.join(LIBDIR, HOOK_NAME)
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall", "-D__HIP_PLATFORM_AMD__",
+           "-I" + os.path.join(rocm, "include"), os.path.join(CSRC, "rccl_hook.cpp"), "-o", hook,
+           "-L" + LIBDIR, "-l:" + LIBNAME, "-L" + os.path.join(rocm, "lib"), "-lamdhip64",
+           "-Wl,-rpath,$ORIGIN", "-ldl", "-lpthread"]
     _run(cmd, verbose)
     return out
 

@@ -1,0 +1,48 @@
+// A stand-in for the part of RCCL that allocates communication buffers through the HIP
+// virtual-memory API, built by tests/test_gpu_rccl_hook.py into a file named librccl_standin.so
+// so that the allocator hook treats its calls as RCCL's. It follows the call order of NCCL's
+// ncclCuMemAlloc / ncclCuMemFree as the reference's patch shows them
+// (nccl_patch/nccl_2.27.5-1.diff:272-296): create, reserve, map, set access; and on free:
+// look the handle up from the address, unmap, release, free the reservation.
+// The RCCL 2.27.7 shipped with ROCm 7.2 never takes this path on its own (its buffers come from
+// plain allocations even with NCCL_CUMEM_ENABLE=1), which is why a stand-in is needed.
+#include <hip/hip_runtime_api.h>
+#include <stddef.h>
+#include <stdint.h>
+
+extern "C" __attribute__((visibility("default"))) int standin_cumem_alloc(void** ptr, size_t size) {
+  hipMemAllocationProp prop = {};
+  prop.type = hipMemAllocationTypePinned;
+  prop.location.type = hipMemLocationTypeDevice;
+  prop.requestedHandleTypes = hipMemHandleTypePosixFileDescriptor;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 1;
+  prop.location.id = dev;
+  size_t gran = 0;
+  if (hipMemGetAllocationGranularity(&gran, &prop, hipMemAllocationGranularityMinimum) != hipSuccess) return 2;
+  if (gran < (2u << 20)) gran = 2u << 20;
+  size = (size + gran - 1) / gran * gran;
+  hipMemGenericAllocationHandle_t handle;
+  if (hipMemCreate(&handle, size, &prop, 0) != hipSuccess) return 3;
+  if (hipMemAddressReserve(ptr, size, gran, nullptr, 0) != hipSuccess) return 4;
+  if (hipMemMap(*ptr, size, 0, handle, 0) != hipSuccess) return 5;
+  hipMemAccessDesc acc = {};
+  acc.location.type = hipMemLocationTypeDevice;
+  acc.location.id = dev;
+  acc.flags = hipMemAccessFlagsProtReadWrite;
+  if (hipMemSetAccess(*ptr, size, &acc, 1) != hipSuccess) return 6;
+  return 0;
+}
+
+extern "C" __attribute__((visibility("default"))) int standin_cumem_free(void* ptr) {
+  hipMemGenericAllocationHandle_t handle = nullptr;
+  // this HIP runtime's retain takes no reference, so there is no release to pair with it
+  if (hipMemRetainAllocationHandle(&handle, ptr) != hipSuccess) return 1;
+  hipDeviceptr_t base = nullptr;
+  size_t size = 0;
+  if (hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)ptr) != hipSuccess) return 2;
+  if (hipMemUnmap(ptr, size) != hipSuccess) return 3;
+  if (hipMemRelease(handle) != hipSuccess) return 4;
+  if (hipMemAddressFree(ptr, size) != hipSuccess) return 5;
+  return 0;
+}

@@ -247,3 +247,14 @@ def test_headers_compile_and_link_from_c_and_cxx(tmp_path):
         r = subprocess.run([out], env=env, capture_output=True, text=True, timeout=60)
         assert r.returncode == 0, (r.returncode, r.stdout[-2000:], r.stderr[-2000:])
         assert "caller ok" in r.stdout
+
+
+def test_rccl_hook_library_exports_the_interposed_calls():
+    hook = os.path.join(os.path.dirname(B.LIB_PATH), "libamem_rccl_hook.so")
+    assert os.path.exists(hook)
+    out = subprocess.run(["nm", "-D", "--defined-only", hook], check=True, capture_output=True, text=True).stdout
+    names = {l.split()[-1] for l in out.splitlines() if " T " in l}
+    assert names == {"hipMemMap", "hipMemSetAccess", "hipMemUnmap", "hipMemImportFromShareableHandle",
+                     "amem_rccl_hook_registered"}
+    # unversioned definitions: they satisfy librccl's versioned references (hipMemMap@hip_5.1 ...)
+    assert "@" not in "".join(names)

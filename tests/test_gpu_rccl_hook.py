@@ -1,0 +1,78 @@
+"""The allocator hook for an unpatched RCCL (libamem_rccl_hook.so): VMM allocations made by a
+library whose file name starts with "librccl" appear in the registry by themselves, survive a
+pause/resume cycle bit-exactly at the same addresses, and disappear from the registry when that
+library frees them. The caller here is a stand-in that allocates the way NCCL's ncclCuMemAlloc
+does; the RCCL build of this ROCm release keeps its own buffers in plain allocations."""
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+CHILD = r'''
+import ctypes as C, os, sys
+import numpy as np
+root, standin = sys.argv[1], sys.argv[2]
+sys.path.insert(0, root)
+libdir = os.path.join(root, "asystem-amem_amd", "lib")
+# order matters: the hook must precede the HIP runtime in the global symbol scope
+hook = C.CDLL(os.path.join(libdir, "libamem_rccl_hook.so"), mode=C.RTLD_GLOBAL)
+from asystem_amem_amd import binding as B, harness as H
+lib = B.load()
+rccl = C.CDLL(standin, mode=C.RTLD_GLOBAL)
+rccl.standin_cumem_alloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+rccl.standin_cumem_free.argtypes = [C.c_void_p]
+hook.amem_rccl_hook_registered.restype = C.c_int64
+MiB = 1 << 20
+rng = np.random.default_rng(31)
+bufs = []
+for k, n in enumerate([4 * MiB, 16 * MiB, 2 * MiB]):
+    p = C.c_void_p()
+    assert rccl.standin_cumem_alloc(C.byref(p), n) == 0
+    data = rng.integers(0, 256, n, dtype=np.uint8)
+    data[n // 4: n // 2] = 0
+    assert lib.amem_copy_to_device(p.value, data.ctypes.data, n) == 0
+    bufs.append((p.value, n, data))
+# the application's own VMM allocation is none of the hook's business
+va, h, asz = C.c_uint64(), C.c_uint64(), C.c_uint64()
+assert lib.amem_vmm_alloc(2 * MiB, 0, C.byref(va), C.byref(h), C.byref(asz)) == 0
+assert lib.amem_region_count(0) == 3 and hook.amem_rccl_hook_registered() == 3
+tab = H.region_table(lib, 0)
+assert sorted(tab) == sorted(b[0] for b in bufs)
+for p, n, _ in bufs:
+    assert tab[p]["alloc_sz"] == n and tab[p]["type"] == B.TYPE_LOCAL and tab[p]["state"] == B.STATE_ALLOC and tab[p]["handle"] != 0
+lib.ncclPause(None); lib.ncclResume(None)                      # warm cycle
+free0 = H.mem_free(lib)
+assert lib.ncclPause(None) == 0 and lib.amem_check_paused(0) == 1
+assert H.mem_free(lib) - free0 >= 22 * MiB - 4 * MiB
+assert lib.ncclResume(None) == 0 and lib.amem_check_paused(0) == 0
+for p, n, data in bufs:
+    out = np.empty(n, dtype=np.uint8)
+    assert lib.amem_copy_from_device(out.ctypes.data, p, n) == 0
+    assert np.array_equal(out, data)
+# the resumed handle is not the one the allocator created; freeing by address still works
+for p, n, _ in bufs[:2]:
+    assert rccl.standin_cumem_free(p) == 0
+assert lib.amem_region_count(0) == 1 and hook.amem_rccl_hook_registered() == 1
+assert lib.ncclPause(None) == 0 and lib.ncclResume(None) == 0
+out = np.empty(bufs[2][1], dtype=np.uint8)
+assert lib.amem_copy_from_device(out.ctypes.data, bufs[2][0], out.nbytes) == 0 and np.array_equal(out, bufs[2][2])
+assert rccl.standin_cumem_free(bufs[2][0]) == 0
+assert lib.amem_region_count(0) == 0 and lib.amem_handle_count(0) == 0
+assert lib.amem_vmm_free(va.value, asz.value, h.value) == 0
+print("rccl hook ok")
+'''
+
+
+def test_hook_registers_and_releases_rccl_style_allocations(gpu, tmp_path):
+    standin = str(tmp_path / "librccl_standin.so")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    subprocess.run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-D__HIP_PLATFORM_AMD__",
+                    "-I" + os.path.join(rocm, "include"), os.path.join(ROOT, "tests", "rccl_standin", "librccl_standin.cpp"),
+                    "-o", standin, "-L" + os.path.join(rocm, "lib"), "-lamdhip64"], check=True, capture_output=True, text=True)
+    env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="1", AMEM_IPC="0")
+    r = subprocess.run([sys.executable, "-c", CHILD, ROOT, standin], env=env, capture_output=True, text=True, timeout=240)
+    assert r.returncode == 0 and "rccl hook ok" in r.stdout, (r.returncode, r.stdout[-3000:], r.stderr[-3000:])
