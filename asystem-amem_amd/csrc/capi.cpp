@@ -577,8 +577,8 @@ static OptRef* opt_table(size_t* n) {
       {"verify", &o.verify, 0, 1},
       {"pause_path", &o.pause_path, 0, 4},
       {"interleave_bytes", &o.interleave_bytes, 1 << 16, (int64_t)1 << 40},
-      {"pause_xcds", &o.pause_xcds, 1, 8},
-      {"pause_wgs", &o.pause_wgs, 1, 65536},
+      {"pause_xcds", &o.pause_xcds, 0, 8},
+      {"pause_wgs", &o.pause_wgs, 0, 65536},
       {"dma_min_bytes", &o.dma_min_bytes, 0, (int64_t)1 << 40},
       {"staging_bytes", &o.staging_bytes, 0, (int64_t)1 << 36},
       {"slab_bytes", &o.slab_bytes, 1 << 16, (int64_t)1 << 36},

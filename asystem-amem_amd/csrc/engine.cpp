@@ -418,6 +418,32 @@ hipError_t Engine::pause_copy_direct(Ctx& c, std::vector<Region*>& regs) {
   return e;
 }
 
+// Launch shape of the interleaved path's gather kernel. Narrow shapes copy more slowly but let
+// the unmaps that run beside them finish sooner; which one ends the pause first depends on how
+// many regions there are per parked byte. Each candidate carries what was measured for it on
+// an MI355X: the rate it sustains while unmaps run beside it, and what one unmap + release then
+// costs. The pause is modelled as the copy time plus, at the idle unmap cost, whatever unmaps
+// did not fit beside the copy.
+struct PauseShape { uint32_t wgs, xcds; double gbps, unmap_ms; };
+static PauseShape choose_pause_shape(uint64_t parked_bytes, size_t regions) {
+  static const PauseShape shapes[] = {
+      {4, 1, 44.0, 0.29},   // 4 workgroups on one XCD
+      {8, 1, 47.0, 0.32},
+      {32, 1, 50.0, 0.42},  // one XCD, saturated
+      {96, 8, 56.0, 2.0},   // the whole chip: fastest copy, unmaps crawl while it runs
+  };
+  const double idle_unmap_ms = 0.26;
+  PauseShape best = shapes[0];
+  double best_ms = 1e300;
+  for (const PauseShape& s : shapes) {
+    const double copy_ms = (double)parked_bytes / (s.gbps * 1e6);
+    const double beside = copy_ms / s.unmap_ms;
+    const double ms = copy_ms + ((double)regions > beside ? ((double)regions - beside) * idle_unmap_ms : 0.0);
+    if (ms < best_ms) { best_ms = ms; best = s; }
+  }
+  return best;
+}
+
 // Interleaved path: the gather kernel writes pinned host memory itself, in many short
 // launches (one per group of regions holding about interleave_bytes of parked data), with an
 // event after each. A second host thread unmaps and releases a group's regions as soon as
@@ -432,6 +458,11 @@ hipError_t Engine::pause_copy_interleaved(Ctx& c, std::vector<Region*>& regs) {
   const uint64_t* tp = (const uint64_t*)h_tiles_.p;
   SlabTable pool_tab = {(uint8_t* const*)d_slabtab_.p, pool_->shift(), pool_->slab_bytes() - 1};
   const uint64_t want = (uint64_t)std::max<int64_t>(options().interleave_bytes, (int64_t)kChunkBytes);
+  PauseShape shape = choose_pause_shape(parked_total_, parked_.size());
+  if (options().pause_wgs > 0) shape.wgs = (uint32_t)options().pause_wgs;      // explicit settings win
+  if (options().pause_xcds > 0) shape.xcds = (uint32_t)options().pause_xcds;
+  LOGGER(DEBUG, "memPause: gather kernel on %u workgroups over %u XCD(s) for %llu MiB in %zu regions", shape.wgs,
+         shape.xcds, (unsigned long long)(parked_total_ >> 20), parked_.size());
   struct Group { size_t r0, r1; uint32_t d0, d1; uint64_t bytes; };
   std::vector<Group> groups;
   const size_t n = parked_.size();
@@ -468,7 +499,7 @@ hipError_t Engine::pause_copy_interleaved(Ctx& c, std::vector<Region*>& regs) {
     if (G.d1 > G.d0 && tp[G.d1] > tp[G.d0]) {
       e = CHECK_HIP(launch_move(false, (const CopyDesc*)d_descs_.p + G.d0, (const uint64_t*)d_tiles_.p + G.d0,
                                 G.d1 - G.d0, tp[G.d0], tp[G.d1] - tp[G.d0], pool_tab, 0,
-                                (uint32_t)options().pause_wgs, (uint32_t)options().pause_xcds, kstream_));
+                                shape.wgs, shape.xcds, kstream_));
       if (e != hipSuccess) break;
       stats_.k2_launches++;
       stats_.kernel_bytes += G.bytes;
