@@ -419,7 +419,13 @@ int amem_mem_pause(int pid, uint64_t tag) {
     return (int)hipErrorNoDevice;
   }
   c->engine = en;
-  return en->pause(*c);
+  bool rolled_back = false;
+  int ret = en->pause(*c, &rolled_back);
+  if (rolled_back) {
+    std::lock_guard<std::mutex> lf(c->fields);
+    c->paused = false;
+  }
+  return ret;
 }
 
 int amem_mem_resume(int pid, uint64_t tag) {
@@ -439,7 +445,9 @@ int amem_mem_resume(int pid, uint64_t tag) {
     Engine* en = engine_for(dev);
     if (!en) return (int)hipErrorNoDevice;
     c->engine = en;
-    ret = en->resume(*c);
+    bool incomplete = false;
+    ret = en->resume(*c, &incomplete);
+    if (incomplete) return ret;  // still paused: a later resume picks up the remaining regions
   }
   std::lock_guard<std::mutex> lf(c->fields);
   c->paused = false;
@@ -588,6 +596,7 @@ static OptRef* opt_table(size_t* n) {
       {"peer_timeout_ms", &o.peer_timeout_ms, 0, (int64_t)1 << 40},
       {"peer_loopback", &o.peer_loopback, 0, 1},
       {"offload_free_tag", &o.offload_free_tag, -1, AMEM_MAX_CALLER - 1},
+      {"pool_limit_bytes", &o.pool_limit_bytes, 0, (int64_t)1 << 46},
   };
   *n = sizeof(t) / sizeof(t[0]);
   return t;

@@ -635,8 +635,9 @@ hipError_t Engine::pause_copy_staged(Ctx& c, std::vector<Region*>& regs, bool* u
   return hipSuccess;
 }
 
-int Engine::pause(Ctx& c) {
+int Engine::pause(Ctx& c, bool* rolled_back) {
   auto t0 = Clock::now();
+  if (rolled_back) *rolled_back = false;
   hipError_t e = init();
   if (e != hipSuccess) return (int)e;
   int rc = 0;
@@ -685,19 +686,6 @@ int Engine::pause(Ctx& c) {
   const int rc_validation = rc;
   rc = 0;  // the valid regions are still paused; the validation error is returned at the end
 
-  // Imported mappings go first (reference step 2, amem_nccl.cpp:517-526): no data to save,
-  // and the owner's release only frees memory once importers have let go.
-  for (auto& pr : imported) {
-    auto tu = Clock::now();
-    Region* r = pr.second;
-    LOGGER(DEBUG, "memPause: release peer handle %llx.", (unsigned long long)pr.first);
-    uint64_t h = r->handle ? r->handle : vmm_handle_of(pr.first);
-    note(vmm_unmap_release(pr.first, r->allocSz, h, 0));
-    std::lock_guard<std::mutex> lk(c.fields);
-    r->state = AMEM_STATE_HOLE;
-    c.releaseShadowCnt++;
-    stats_.pause_unmap_ms += ms_since(tu);
-  }
   stats_.peer_regions = imported.size();
   stats_.local_regions = locals.size();
 
@@ -758,9 +746,42 @@ int Engine::pause(Ctx& c) {
   parked_total_ = cursor;
   stats_.parked_bytes = cursor;
   stats_.zero_chunks = zero_chunks;
-  e = pool_->ensure(cursor);
+  const uint64_t limit = (uint64_t)options().pool_limit_bytes;
+  if (limit && cursor > limit) {
+    LOGGER(ERROR, "memPause: groupID:%d pid:%d GPU:%d needs %llu MiB of pinned host memory, the limit is %llu MiB",
+           amem_groupID_value(), getpid(), dev_, (unsigned long long)(cursor >> 20), (unsigned long long)(limit >> 20));
+    e = hipErrorOutOfMemory;
+  } else {
+    e = pool_->ensure(cursor);
+  }
   note(e);
   stats_.slab_bytes = pool_->capacity();
+  if (rc != 0) {
+    // Nothing has been copied, unmapped or released yet: undo the bookkeeping and report.
+    // The caller is not paused.
+    std::lock_guard<std::mutex> lk(c.fields);
+    for (Region* r : locals) { r->state = AMEM_STATE_ALLOC; c.offloadCnt--; }
+    parked_.clear();
+    gather_descs_.clear();
+    LOGGER(ERROR, "memPause: groupID:%d pid:%d GPU:%d failed with HIP error %d before anything was released; "
+           "the process is not paused", amem_groupID_value(), getpid(), dev_, rc);
+    if (rolled_back) *rolled_back = true;
+    return rc;
+  }
+
+  // Imported mappings go before the local ones (reference step 2, amem_nccl.cpp:517-526): no
+  // data to save, and the owner's release only frees memory once importers have let go.
+  for (auto& pr : imported) {
+    auto tu = Clock::now();
+    Region* r = pr.second;
+    LOGGER(DEBUG, "memPause: release peer handle %llx.", (unsigned long long)pr.first);
+    uint64_t h = r->handle ? r->handle : vmm_handle_of(pr.first);
+    note(vmm_unmap_release(pr.first, r->allocSz, h, 0));
+    std::lock_guard<std::mutex> lk(c.fields);
+    r->state = AMEM_STATE_HOLE;
+    c.releaseShadowCnt++;
+    stats_.pause_unmap_ms += ms_since(tu);
+  }
   for (size_t i = 0; i < locals.size(); ++i) {
     locals[i]->parkedBytes = parked_[i].parked_bytes;
     locals[i]->cpuAddr = (parked_[i].parked_bytes && e == hipSuccess) ? pool_->host_addr(parked_[i].parked_off) : nullptr;
@@ -822,7 +843,8 @@ void Engine::forget(uint64_t va) {
 // resume
 // ---------------------------------------------------------------------------------------
 
-int Engine::resume(Ctx& c) {
+int Engine::resume(Ctx& c, bool* incomplete) {
+  if (incomplete) *incomplete = false;
   hipError_t e = init();
   if (e != hipSuccess) return (int)e;
   int rc = 0;
@@ -836,6 +858,16 @@ int Engine::resume(Ctx& c) {
   stats_.resume_ms = stats_.resume_map_ms = stats_.resume_copy_ms = stats_.resume_peer_ms = 0;
   stats_.k3_ms = 0; stats_.k3_launches = 0; stats_.verify_mismatch = 0;
   auto& table = c.allocTable[dev_];
+
+  // A pause that failed half-way leaves regions it never released in OFFLOADING: they still
+  // have their memory and their bytes.
+  {
+    std::lock_guard<std::mutex> lk(c.fields);
+    for (auto& kv : table) {
+      Region& r = kv.second;
+      if (!from_peer(r.type) && r.state == AMEM_STATE_OFFLOADING) { r.state = AMEM_STATE_ALLOC; c.offloadCnt--; }
+    }
+  }
 
   // Scatter list: per region, its parked runs and its zero runs.
   struct Item { Region* r; uint64_t va; uint32_t d0, d1; uint64_t bytes; };
@@ -1023,6 +1055,19 @@ int Engine::resume(Ctx& c) {
     }
   }
   stats_.resume_peer_ms = ms_since(tpeer);
+  if (rc != 0) {
+    // Regions still without memory keep their parked bytes: the caller stays paused and may
+    // call resume again, e.g. once device memory another process held has been given back.
+    size_t holes = 0;
+    std::lock_guard<std::mutex> lk(c.fields);
+    for (auto& kv : table) holes += kv.second.state == AMEM_STATE_HOLE && !from_peer(kv.second.type);
+    // (an import still waiting for its owner is remapped by the service thread whenever the owner re-exports)
+    if (holes) {
+      LOGGER(ERROR, "memResume: groupID:%d pid:%d GPU:%d failed with error %d, %zu local regions are still released; "
+             "the process stays paused and resume can be called again", amem_groupID_value(), getpid(), dev_, rc, holes);
+      if (incomplete) *incomplete = true;
+    }
+  }
   stats_.resume_ms = ms_since(t0);
   (void)CHECK_HIP(hipMemGetInfo(&free_sz, &total));
   LOGGER(INFO, "groupID:%d pid:%d GPU:%d resumeCnt:%ld memUsed:%ld MB after resumed, duration:%ld ms "

@@ -30,6 +30,7 @@ struct Options {
   int64_t hbm_wgs = 65536;                // workgroup cap of device-only kernels
   int64_t resume_batch_bytes = 64ll << 20;
   int64_t peer_timeout_ms = 60000;
+  int64_t pool_limit_bytes = 0;           // cap on pinned host memory a pause may need, 0 = none
   int64_t offload_free_tag = -1;          // caller tag whose regions are released without being copied
   int64_t peer_loopback = 0;              // let a process register with / update its own service (tests)
 };
@@ -67,8 +68,10 @@ class Engine {
   hipError_t init();
 
   // Both are called with Ctx::structure held.
-  int pause(Ctx& c);
-  int resume(Ctx& c);
+  // *rolled_back is set when the pause failed before releasing anything and undid itself.
+  int pause(Ctx& c, bool* rolled_back);
+  // *incomplete is set when regions are still released after a failed resume (retry possible).
+  int resume(Ctx& c, bool* incomplete);
   // A region was deleted while paused: drop its parked bytes.
   void forget(uint64_t va);
 

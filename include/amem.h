@@ -282,6 +282,9 @@ int amem_set_enabled(int on);
  *                     AMEM_NCCL_OFFLOAD_FREE_TAG is documented to do in the reference, where the
  *                     variable is parsed but never takes effect (amem_nccl.cpp:40, :503, :620);
  *                     the environment variable stays ineffective here too, only this option acts
+ *   "pool_limit_bytes" most pinned host memory one pause may need (0 = no limit). A pause that
+ *                     would need more fails with an out-of-memory error before it has released
+ *                     anything, and the process stays un-paused
  *   "peer_loopback"   0/1   treat this process's own slot like any other peer: registration and
  *                     re-export go through the socket service of the same process (default 0:
  *                     a process never registers with itself, gmm_client_impl.cpp:482-484, :512-514) */

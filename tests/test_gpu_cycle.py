@@ -13,6 +13,7 @@ from asystem_amem_amd.footprint import CHUNK, Footprint
 
 pytestmark = pytest.mark.gpu
 MiB = 1 << 20
+GiB = 1 << 30
 
 
 @pytest.fixture()
@@ -319,3 +320,68 @@ def test_stale_registration_is_reported_not_read(eng):
     ext = (B.Extent * 1)(B.Extent(0x7e0000000000, 65536))
     one = (C.c_uint8 * 1)()
     assert lib.amem_zero_scan(ext, 1, one, None, None) != 0
+
+
+def test_pause_that_cannot_park_its_bytes_rolls_back(eng):
+    """Host memory for the parked bytes is capped: the pause must fail before it releases
+    anything, leave the process un-paused with every region mapped and intact, and succeed
+    once the cap is lifted. The failure is forced from the host; the GPU does nothing unusual."""
+    lib = eng
+    fp = Footprint(2, 13, max_regions=8, threads=4)              # 32 MiB, about half of it non-zero
+    regs = H.Regions(lib, fp)
+    assert lib.amem_mem_pause(0, 0) == 0 and lib.amem_mem_resume(0, 0) == 0   # engine scratch now exists
+    before, c0 = regs.table(), H.counters(lib)
+    assert lib.amem_set_option(b"pool_limit_bytes", 4 * MiB) == 0
+    try:
+        free0 = H.mem_free(lib)
+        assert lib.amem_mem_pause(0, 0) != 0
+        assert lib.amem_check_paused(0) == 0
+        c = H.counters(lib)
+        assert c == c0
+        assert regs.table() == before                                # handles, states, everything
+        assert abs(H.mem_free(lib) - free0) < 2 * MiB
+        assert regs.mismatched_bytes() == 0
+        assert lib.amem_mem_resume(0, 0) == 0                         # not paused: no-op
+    finally:
+        assert lib.amem_set_option(b"pool_limit_bytes", 0) == 0
+    assert lib.amem_mem_pause(0, 0) == 0 and lib.amem_mem_resume(0, 0) == 0
+    assert regs.mismatched_bytes() == 0
+    regs.free()
+
+
+def test_resume_without_enough_device_memory_can_be_retried(eng):
+    """The memory a pause gave up may be in use by someone else when resume is called. Resume then
+    fails with an out-of-memory error, keeps the parked bytes and stays paused; once the memory is
+    back a second resume restores every region bit for bit. The shortage is made from the host by
+    allocating the free device memory; no kernel is involved in the failure."""
+    lib = eng
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+    hip.hipFree.argtypes = [C.c_void_p]
+    fp = Footprint(1, 17, max_regions=24, threads=8)             # 24 regions, a few hundred MiB
+    regs = H.Regions(lib, fp)
+    assert lib.amem_mem_pause(0, 0) == 0
+    # leave less than the footprint: some regions get memory, the rest cannot. The free figure
+    # the runtime reports is only approximate, so top up in small blocks until it reads low enough.
+    hogs = [C.c_void_p()]
+    assert hip.hipMalloc(C.byref(hogs[0]), H.mem_free(lib) - 2 * GiB) == 0
+    while H.mem_free(lib) > int(fp.total_bytes) // 2 and len(hogs) < 200:
+        hogs.append(C.c_void_p())
+        assert hip.hipMalloc(C.byref(hogs[-1]), 32 * MiB) == 0
+    try:
+        rc = lib.amem_mem_resume(0, 0)
+        assert rc != 0
+        c = H.counters(lib)
+        assert c["paused"] == 1 and c["resume_cnt"] == 0 and c["offload_cnt"] > 0
+        states = [r["state"] for r in regs.table().values()]
+        assert B.STATE_HOLE in states and B.STATE_PRELOADING not in states
+    finally:
+        for hog in hogs:
+            assert hip.hipFree(hog) == 0
+    assert lib.amem_mem_resume(0, 0) == 0
+    c = H.counters(lib)
+    assert c["paused"] == 0 and c["offload_cnt"] == 0
+    assert regs.mismatched_bytes() == 0
+    assert lib.amem_mem_pause(0, 0) == 0 and lib.amem_mem_resume(0, 0) == 0      # and the next cycle is ordinary
+    assert regs.mismatched_bytes() == 0
+    regs.free()
