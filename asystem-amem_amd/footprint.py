@@ -120,3 +120,42 @@ class Footprint:
 
     def zero_chunks(self):
         return int(self.mask[:self.nchunks].sum())
+
+
+class PackedGranules:
+    """Configuration 4 as an allocator sees it: the sub-allocations of a Footprint(4, ...) bump-packed
+    into 2 MiB granules (none straddles a granule; the gaps read zero). Each granule is one region.
+    Offers the part of Footprint's interface that harness.Regions uses."""
+
+    GRANULE = 2 << 20
+
+    def __init__(self, seed=3, count=100000, threads=8):
+        self.sub = Footprint(4, seed, max_regions=count, threads=threads)
+        g = self.GRANULE
+        sz = self.sub.sizes.astype(np.int64)
+        self.starts = np.zeros(len(sz), dtype=np.int64)
+        cur = 0
+        for i, n in enumerate(sz):
+            if cur % g + n > g:
+                cur = (cur // g + 1) * g
+            self.starts[i] = cur
+            cur += int(n)
+        self.ngranules = (cur + g - 1) // g
+        self.sizes = np.full(self.ngranules, g, dtype=np.uint64)
+        self.total_bytes = int(self.ngranules) * g
+        self.payload_bytes = int(sz.sum())
+        # sub-allocations of granule k: [first[k], first[k + 1])
+        self.first = np.searchsorted(self.starts // g, np.arange(self.ngranules + 1), side="left")
+
+    def region_bytes(self, i, out=None):
+        g = self.GRANULE
+        if out is None:
+            out = np.empty(g, dtype=np.uint8)
+        out[:g] = 0
+        for s in range(int(self.first[i]), int(self.first[i + 1])):
+            a = int(self.starts[s]) - i * g
+            self.sub.region_bytes(s, out[a:a + int(self.sub.sizes[s])])
+        return out[:g]
+
+    def check_region(self, i, buf):
+        return int(np.count_nonzero(buf[:self.GRANULE] != self.region_bytes(i)))

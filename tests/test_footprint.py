@@ -100,3 +100,24 @@ def test_mutation_changes_both_ways():
     for c in range(f.nchunks):
         same = np.array_equal(before[c], f.chunk_bytes(c))
         assert same == (c not in set(int(t) for t in touched)) or (before_mask[c] and f.mask[c])
+
+
+def test_packed_granules_layout():
+    """Configuration 4's sub-allocations inside 2 MiB granules: none straddles a granule, every byte of a
+    granule is either the sub-allocation's own stream or a zero gap, and the check finds a flipped byte."""
+    pg = F.PackedGranules(3, 400, threads=2)
+    g = pg.GRANULE
+    ends = pg.starts + pg.sub.sizes.astype(np.int64)
+    assert (pg.starts // g == (ends - 1) // g).all() and (pg.starts[1:] >= ends[:-1]).all()
+    assert pg.ngranules == ends[-1] // g + (ends[-1] % g != 0) and pg.payload_bytes == int(pg.sub.sizes.sum())
+    k = pg.ngranules // 2
+    img = pg.region_bytes(k).copy()
+    live = np.zeros(g, dtype=bool)
+    for s in range(int(pg.first[k]), int(pg.first[k + 1])):
+        a, n = int(pg.starts[s]) - k * g, int(pg.sub.sizes[s])
+        assert np.array_equal(img[a:a + n], pg.sub.region_bytes(s))
+        live[a:a + n] = True
+    assert int(pg.first[k + 1]) > int(pg.first[k]) and not img[~live].any()
+    assert pg.check_region(k, img) == 0
+    img[12345] ^= 1
+    assert pg.check_region(k, img) == 1

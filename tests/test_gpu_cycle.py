@@ -9,7 +9,7 @@ import pytest
 import oracle as O
 from asystem_amem_amd import binding as B
 from asystem_amem_amd import harness as H
-from asystem_amem_amd.footprint import CHUNK, Footprint
+from asystem_amem_amd.footprint import CHUNK, Footprint, PackedGranules
 
 pytestmark = pytest.mark.gpu
 MiB = 1 << 20
@@ -383,5 +383,25 @@ def test_resume_without_enough_device_memory_can_be_retried(eng):
     assert c["paused"] == 0 and c["offload_cnt"] == 0
     assert regs.mismatched_bytes() == 0
     assert lib.amem_mem_pause(0, 0) == 0 and lib.amem_mem_resume(0, 0) == 0      # and the next cycle is ordinary
+    assert regs.mismatched_bytes() == 0
+    regs.free()
+
+
+def test_config4_packed_granules_cycle(eng):
+    """benchmark configuration 4 at full size: 100,000 sub-allocations of 4-64 KiB (seed 3) bump-packed
+    into about a thousand 2 MiB granules, every granule one tracked region. Many small regions make
+    the per-region costs dominate; the bytes and the table must come back all the same."""
+    lib = eng
+    fp = PackedGranules(3, 100000, threads=8)
+    assert 900 < fp.ngranules < 1100 and fp.payload_bytes > 0.95 * fp.total_bytes
+    regs = H.Regions(lib, fp)
+    before = regs.table()
+    free0 = H.mem_free(lib)
+    assert lib.amem_mem_pause(0, 0) == 0
+    assert H.mem_free(lib) - free0 > 0.95 * fp.total_bytes
+    assert lib.amem_mem_resume(0, 0) == 0
+    st = H.cycle_stats(lib)
+    assert st["local_regions"] == fp.ngranules and st["footprint_bytes"] == fp.total_bytes
+    assert H.compare_tables(before, regs.table()) == []
     assert regs.mismatched_bytes() == 0
     regs.free()
