@@ -54,6 +54,9 @@ static Ctx* init_ctx(int dev) {
     g.ctx = new Ctx();
     const char* ipc = getenv("AMEM_IPC");
     if (!ipc || atoi(ipc) != 0) (void)ipc_start(dev);
+    // Streams and device code are set up while there is still device memory to load them into.
+    // (the current device: pause and resume act on it, and selecting it changes nothing for the caller)
+    if (gpu_present()) (void)engine_for(current_device());
   }
   return g.ctx;
 }
@@ -597,6 +600,7 @@ static OptRef* opt_table(size_t* n) {
       {"peer_loopback", &o.peer_loopback, 0, 1},
       {"offload_free_tag", &o.offload_free_tag, -1, AMEM_MAX_CALLER - 1},
       {"pool_limit_bytes", &o.pool_limit_bytes, 0, (int64_t)1 << 46},
+      {"scratch_on_host", &o.scratch_on_host, 0, 1},
   };
   *n = sizeof(t) / sizeof(t[0]);
   return t;

@@ -25,18 +25,32 @@ Options& options() {
   return o;
 }
 
-hipError_t DevBuf::ensure(size_t bytes) {
-  if (bytes <= cap) return hipSuccess;
+// Pause is called when device memory is short, possibly gone. Scratch that does not fit on
+// the device goes to pinned host memory, which the kernels reach over the link: slower
+// table lookups, same results.
+hipError_t DevBuf::ensure(size_t bytes, bool grow_on_host) {
+  const bool forced = options().scratch_on_host != 0;
+  if (bytes <= cap && (!forced || host)) return hipSuccess;
+  const bool want_host = forced || grow_on_host;
   release();
   size_t want = std::max<size_t>(bytes + bytes / 4, 4096);
-  hipError_t e = CHECK_HIP(hipMalloc(&p, want));
-  if (e != hipSuccess) { p = nullptr; return e; }
+  if (!want_host) {
+    if (hipMalloc(&p, want) == hipSuccess) { cap = want; return hipSuccess; }
+    (void)hipGetLastError();
+    p = nullptr;
+    LOGGER(WARN, "no device memory for %zu KiB of engine scratch, placing it in pinned host memory", want >> 10);
+  }
+  hipError_t e = CHECK_HIP(hipHostMalloc(&host, want, hipHostMallocDefault));
+  if (e != hipSuccess) { host = nullptr; return e; }
+  e = CHECK_HIP(hipHostGetDevicePointer(&p, host, 0));
+  if (e != hipSuccess) { (void)hipHostFree(host); host = p = nullptr; return e; }
   cap = want;
   return hipSuccess;
 }
 void DevBuf::release() {
-  if (p) (void)CHECK_HIP(hipFree(p));
-  p = nullptr;
+  if (host) (void)CHECK_HIP(hipHostFree(host));
+  else if (p) (void)CHECK_HIP(hipFree(p));
+  p = host = nullptr;
   cap = 0;
 }
 hipError_t PinBuf::ensure(size_t bytes) {
@@ -78,6 +92,9 @@ hipError_t Engine::init() {
   e = CHECK_HIP(hipStreamCreateWithFlags(&kstream_, hipStreamNonBlocking));
   if (e != hipSuccess) return e;
   e = CHECK_HIP(hipStreamCreateWithFlags(&dstream_, hipStreamNonBlocking));
+  if (e != hipSuccess) return e;
+  // Load the kernels' code now: at the first pause there may be no device memory left for it.
+  e = CHECK_HIP(preload_kernels());
   if (e != hipSuccess) return e;
   pool_ = new SlabPool((uint64_t)options().slab_bytes);
   inited_ = true;
@@ -121,16 +138,16 @@ hipError_t Engine::run_scan(const std::vector<ScanSeg>& segs, uint64_t* nchunks_
   prefix[n] = total;
   *nchunks_out = total;
   if (total == 0) { if (ms) *ms = 0; return hipSuccess; }
-  if ((e = d_segs_.ensure(n * sizeof(ScanSeg))) != hipSuccess) return e;
-  if ((e = d_prefix_.ensure((n + 1) * sizeof(uint64_t))) != hipSuccess) return e;
-  if ((e = d_flags_.ensure(total)) != hipSuccess) return e;
+  if ((e = d_segs_.ensure(n * sizeof(ScanSeg), grow_on_host_)) != hipSuccess) return e;
+  if ((e = d_prefix_.ensure((n + 1) * sizeof(uint64_t), grow_on_host_)) != hipSuccess) return e;
+  if ((e = d_flags_.ensure(total, grow_on_host_)) != hipSuccess) return e;
   if ((e = h_flags_.ensure(total)) != hipSuccess) return e;
   if (want_sums) {
-    if ((e = d_sums_.ensure(total * sizeof(ChunkSum))) != hipSuccess) return e;
+    if ((e = d_sums_.ensure(total * sizeof(ChunkSum), grow_on_host_)) != hipSuccess) return e;
   }
-  e = CHECK_HIP(hipMemcpyAsync(d_segs_.p, h_segs_.p, n * sizeof(ScanSeg), hipMemcpyHostToDevice, kstream_));
+  e = CHECK_HIP(hipMemcpyAsync(d_segs_.p, h_segs_.p, n * sizeof(ScanSeg), hipMemcpyDefault, kstream_));
   if (e != hipSuccess) return e;
-  e = CHECK_HIP(hipMemcpyAsync(d_prefix_.p, h_prefix_.p, (n + 1) * sizeof(uint64_t), hipMemcpyHostToDevice, kstream_));
+  e = CHECK_HIP(hipMemcpyAsync(d_prefix_.p, h_prefix_.p, (n + 1) * sizeof(uint64_t), hipMemcpyDefault, kstream_));
   if (e != hipSuccess) return e;
   hipEvent_t e0 = event_at(0), e1 = event_at(1);
   (void)CHECK_HIP(hipEventRecord(e0, kstream_));
@@ -139,7 +156,7 @@ hipError_t Engine::run_scan(const std::vector<ScanSeg>& segs, uint64_t* nchunks_
                             (uint32_t)options().hbm_wgs, kstream_));
   if (e != hipSuccess) return e;
   (void)CHECK_HIP(hipEventRecord(e1, kstream_));
-  e = CHECK_HIP(hipMemcpyAsync(h_flags_.p, d_flags_.p, total, hipMemcpyDeviceToHost, kstream_));
+  e = CHECK_HIP(hipMemcpyAsync(h_flags_.p, d_flags_.p, total, hipMemcpyDefault, kstream_));
   if (e != hipSuccess) return e;
   e = CHECK_HIP(hipStreamSynchronize(kstream_));
   if (e != hipSuccess) return e;
@@ -178,7 +195,7 @@ hipError_t Engine::zero_scan(const amem_extent* ext, uint64_t n, uint8_t* flags,
   if (e != hipSuccess || total == 0) return e;
   memcpy(flags, h_flags_.p, total);
   if (sums) {
-    e = CHECK_HIP(hipMemcpy(sums, d_sums_.p, total * sizeof(ChunkSum), hipMemcpyDeviceToHost));
+    e = CHECK_HIP(hipMemcpy(sums, d_sums_.p, total * sizeof(ChunkSum), hipMemcpyDefault));
   }
   return e;
 }
@@ -187,12 +204,20 @@ hipError_t Engine::zero_scan(const amem_extent* ext, uint64_t n, uint8_t* flags,
 // descriptor plumbing
 // ---------------------------------------------------------------------------------------
 
+hipError_t Engine::reserve_descs(size_t n) {
+  hipError_t e;
+  if ((e = h_descs_.ensure(std::max<size_t>(n, 1) * sizeof(CopyDesc))) != hipSuccess) return e;
+  if ((e = h_tiles_.ensure((n + 1) * sizeof(uint64_t))) != hipSuccess) return e;
+  if ((e = d_descs_.ensure(std::max<size_t>(n, 1) * sizeof(CopyDesc), grow_on_host_)) != hipSuccess) return e;
+  return d_tiles_.ensure((n + 1) * sizeof(uint64_t), grow_on_host_);
+}
+
 hipError_t Engine::upload_descs(const CopyDesc* descs, size_t n, uint64_t* ntiles_out) {
   hipError_t e;
   if ((e = h_descs_.ensure(std::max<size_t>(n, 1) * sizeof(CopyDesc))) != hipSuccess) return e;
   if ((e = h_tiles_.ensure((n + 1) * sizeof(uint64_t))) != hipSuccess) return e;
-  if ((e = d_descs_.ensure(std::max<size_t>(n, 1) * sizeof(CopyDesc))) != hipSuccess) return e;
-  if ((e = d_tiles_.ensure((n + 1) * sizeof(uint64_t))) != hipSuccess) return e;
+  if ((e = d_descs_.ensure(std::max<size_t>(n, 1) * sizeof(CopyDesc), grow_on_host_)) != hipSuccess) return e;
+  if ((e = d_tiles_.ensure((n + 1) * sizeof(uint64_t), grow_on_host_)) != hipSuccess) return e;
   uint64_t* tp = (uint64_t*)h_tiles_.p;
   uint64_t tiles = 0;
   for (size_t i = 0; i < n; ++i) {
@@ -203,10 +228,10 @@ hipError_t Engine::upload_descs(const CopyDesc* descs, size_t n, uint64_t* ntile
   *ntiles_out = tiles;
   if (n) memcpy(h_descs_.p, descs, n * sizeof(CopyDesc));
   if (n) {
-    e = CHECK_HIP(hipMemcpyAsync(d_descs_.p, h_descs_.p, n * sizeof(CopyDesc), hipMemcpyHostToDevice, kstream_));
+    e = CHECK_HIP(hipMemcpyAsync(d_descs_.p, h_descs_.p, n * sizeof(CopyDesc), hipMemcpyDefault, kstream_));
     if (e != hipSuccess) return e;
   }
-  return CHECK_HIP(hipMemcpyAsync(d_tiles_.p, h_tiles_.p, (n + 1) * sizeof(uint64_t), hipMemcpyHostToDevice, kstream_));
+  return CHECK_HIP(hipMemcpyAsync(d_tiles_.p, h_tiles_.p, (n + 1) * sizeof(uint64_t), hipMemcpyDefault, kstream_));
 }
 
 // Device-side table of contiguous-side base addresses: pool slabs first, then the two
@@ -216,7 +241,7 @@ hipError_t Engine::upload_slab_table() {
   const size_t entries = ns + 3;
   hipError_t e;
   if ((e = h_slabtab_.ensure(entries * sizeof(void*))) != hipSuccess) return e;
-  if ((e = d_slabtab_.ensure(entries * sizeof(void*))) != hipSuccess) return e;
+  if ((e = d_slabtab_.ensure(entries * sizeof(void*), grow_on_host_)) != hipSuccess) return e;
   uint8_t** tab = (uint8_t**)h_slabtab_.p;
   for (size_t i = 0; i < ns; ++i) {
     void* dp = nullptr;
@@ -228,7 +253,7 @@ hipError_t Engine::upload_slab_table() {
   tab[ns + 1] = (uint8_t*)d_staging_[1].p;
   tab[ns + 2] = nullptr;
   slab_table_count_ = ns;
-  return CHECK_HIP(hipMemcpyAsync(d_slabtab_.p, h_slabtab_.p, entries * sizeof(void*), hipMemcpyHostToDevice, kstream_));
+  return CHECK_HIP(hipMemcpyAsync(d_slabtab_.p, h_slabtab_.p, entries * sizeof(void*), hipMemcpyDefault, kstream_));
 }
 
 // Append `d`, cut where its contiguous side would cross a slab boundary.
@@ -245,7 +270,7 @@ static void push_split(std::vector<CopyDesc>& out, CopyDesc d, uint64_t slab_byt
 // offsets from *cursor; zero runs are emitted only when `zero_out` is given.
 static void emit_runs(const uint8_t* flags, uint64_t va, uint64_t size, bool elide, uint64_t* cursor,
                       uint64_t slab_bytes, std::vector<CopyDesc>* data_out,
-                      std::vector<CopyDesc>* zero_out, uint64_t* zero_chunks) {
+                      std::vector<CopyDesc>* zero_out, uint64_t* zero_chunks, uint64_t* zero_runs = nullptr) {
   const uint64_t n = chunks_of(size);
   uint64_t k = 0;
   while (k < n) {
@@ -256,6 +281,7 @@ static void emit_runs(const uint8_t* flags, uint64_t va, uint64_t size, bool eli
     const uint64_t end = std::min(size, j * kChunkBytes);
     if (z) {
       if (zero_chunks) *zero_chunks += j - k;
+      if (zero_runs) ++*zero_runs;
       if (zero_out) zero_out->push_back({va + start, kDescZero, end - start});
     } else {
       if (data_out) push_split(*data_out, {va + start, *cursor, end - start}, slab_bytes);
@@ -300,7 +326,7 @@ hipError_t Engine::move(bool scatter, const amem_copy_desc* descs, uint64_t n, v
   const size_t spare = pool_->slab_count() + 2;
   ((uint8_t**)h_slabtab_.p)[spare] = (uint8_t*)dp;
   e = CHECK_HIP(hipMemcpyAsync((uint8_t**)d_slabtab_.p + spare, (uint8_t**)h_slabtab_.p + spare,
-                               sizeof(void*), hipMemcpyHostToDevice, kstream_));
+                               sizeof(void*), hipMemcpyDefault, kstream_));
   if (e != hipSuccess) return e;
   SlabTable st = {(uint8_t* const*)d_slabtab_.p + spare, 63, ~(uint64_t)0 >> 1};
   hipEvent_t e0 = event_at(0), e1 = event_at(1);
@@ -485,7 +511,8 @@ hipError_t Engine::pause_copy_interleaved(Ctx& c, std::vector<Region*>& regs) {
         if (failed.load()) return;
         std::this_thread::yield();
       }
-      if (hipEventSynchronize(events_[ev0 + g]) != hipSuccess) { failed.store((int)hipGetLastError()); return; }
+      hipError_t es2 = CHECK_HIP(hipEventSynchronize(events_[ev0 + g]));
+      if (es2 != hipSuccess) { failed.store((int)es2); return; }
       for (size_t r = groups[g].r0; r < groups[g].r1; ++r) {
         hipError_t e2 = release_local(c, regs[r], parked_[r].va);
         if (e2 != hipSuccess) { failed.store((int)e2); return; }
@@ -642,6 +669,12 @@ int Engine::pause(Ctx& c, bool* rolled_back) {
   if (e != hipSuccess) return (int)e;
   int rc = 0;
   auto note = [&](hipError_t x) { if (x != hipSuccess && rc == 0) rc = (int)x; };
+  // Tables that an earlier cycle had to place in host memory get another chance on the device.
+  if (!options().scratch_on_host) {
+    DevBuf* db[] = {&d_segs_, &d_prefix_, &d_flags_, &d_sums_, &d_descs_, &d_tiles_, &d_slabtab_};
+    for (DevBuf* b : db) if (b->host) b->release();
+  }
+  grow_on_host_ = false;
   const int64_t path = options().pause_path;
   ref_mode_ = (path == 4);
   const bool elide = options().zero_elide != 0 && !ref_mode_;
@@ -694,6 +727,18 @@ int Engine::pause(Ctx& c, bool* rolled_back) {
     std::lock_guard<std::mutex> lk(c.fields);
     for (Region* r : locals) { r->state = AMEM_STATE_OFFLOADING; c.offloadCnt++; }
   }
+  // Until the copy starts nothing has been copied, unmapped or released: a failure undoes the
+  // bookkeeping and reports, and the caller is not paused.
+  auto undo = [&]() {
+    std::lock_guard<std::mutex> lk(c.fields);
+    for (Region* r : locals) { r->state = AMEM_STATE_ALLOC; c.offloadCnt--; }
+    parked_.clear();
+    gather_descs_.clear();
+    LOGGER(ERROR, "memPause: groupID:%d pid:%d GPU:%d failed with HIP error %d before anything was released; "
+           "the process is not paused", amem_groupID_value(), getpid(), dev_, rc);
+    if (rolled_back) *rolled_back = true;
+    return rc;
+  };
   auto ts = Clock::now();
   float k1ms = 0;
   have_sums_ = !ref_mode_;
@@ -708,8 +753,9 @@ int Engine::pause(Ctx& c, bool* rolled_back) {
   note(e);
   if (e == hipSuccess && nchunks_ && !ref_mode_) {
     note(h_sums_.ensure(nchunks_ * sizeof(ChunkSum)));
-    note(CHECK_HIP(hipMemcpyAsync(h_sums_.p, d_sums_.p, nchunks_ * sizeof(ChunkSum), hipMemcpyDeviceToHost, kstream_)));
+    note(CHECK_HIP(hipMemcpyAsync(h_sums_.p, d_sums_.p, nchunks_ * sizeof(ChunkSum), hipMemcpyDefault, kstream_)));
   }
+  if (rc != 0) return undo();
   stats_.k1_ms = k1ms;
   stats_.k1_launches = (nchunks_ && !ref_mode_) ? 1 : 0;
   stats_.pause_scan_ms = ms_since(ts);
@@ -719,7 +765,7 @@ int Engine::pause(Ctx& c, bool* rolled_back) {
   stats_.total_chunks = nchunks_;
 
   auto tp = Clock::now();
-  uint64_t cursor = 0, chunk0 = 0, zero_chunks = 0;
+  uint64_t cursor = 0, chunk0 = 0, zero_chunks = 0, zero_runs = 0;
   const uint8_t* flags = parked_flags_.data();
   uint64_t slab_bytes = pool_->slab_bytes();
   for (size_t i = 0; i < locals.size(); ++i) {
@@ -736,7 +782,7 @@ int Engine::pause(Ctx& c, bool* rolled_back) {
     p.skip = !ref_mode_ && options().offload_free_tag >= 0 && (int64_t)locals[i]->tags == options().offload_free_tag;
     if (p.skip) std::fill(parked_flags_.begin() + chunk0, parked_flags_.begin() + chunk0 + p.nchunks, (uint8_t)1);
     emit_runs(flags + chunk0, p.va, p.size, elide || p.skip, &cursor, slab_bytes, &gather_descs_, nullptr,
-              p.skip ? nullptr : &zero_chunks);
+              p.skip ? nullptr : &zero_chunks, &zero_runs);
     p.desc_end = (uint32_t)gather_descs_.size();
     p.parked_bytes = cursor - p.parked_off;
     chunk0 += p.nchunks;
@@ -755,19 +801,12 @@ int Engine::pause(Ctx& c, bool* rolled_back) {
     e = pool_->ensure(cursor);
   }
   note(e);
+  // Resume's scatter list is the gather list plus the zero runs (plus one entry per region that
+  // was never saved). Its tables are sized now: what resume has to allocate must not come out of
+  // the device memory the regions are about to give up.
+  note(reserve_descs(gather_descs_.size() + zero_runs + table.size()));
   stats_.slab_bytes = pool_->capacity();
-  if (rc != 0) {
-    // Nothing has been copied, unmapped or released yet: undo the bookkeeping and report.
-    // The caller is not paused.
-    std::lock_guard<std::mutex> lk(c.fields);
-    for (Region* r : locals) { r->state = AMEM_STATE_ALLOC; c.offloadCnt--; }
-    parked_.clear();
-    gather_descs_.clear();
-    LOGGER(ERROR, "memPause: groupID:%d pid:%d GPU:%d failed with HIP error %d before anything was released; "
-           "the process is not paused", amem_groupID_value(), getpid(), dev_, rc);
-    if (rolled_back) *rolled_back = true;
-    return rc;
-  }
+  if (rc != 0) return undo();
 
   // Imported mappings go before the local ones (reference step 2, amem_nccl.cpp:517-526): no
   // data to save, and the owner's release only frees memory once importers have let go.
@@ -850,6 +889,10 @@ int Engine::resume(Ctx& c, bool* incomplete) {
   int rc = 0;
   auto note = [&](hipError_t x) { if (x != hipSuccess && rc == 0) rc = (int)x; };
   const bool elide = elide_used_;
+  // Device memory is spoken for while paused: the regions need back exactly what they gave up.
+  // Anything the engine still has to allocate goes to host memory.
+  grow_on_host_ = true;
+  struct Restore { bool& b; ~Restore() { b = false; } } restore_growth{grow_on_host_};
   size_t free_sz = 0, total = 0;
   (void)CHECK_HIP(hipMemGetInfo(&free_sz, &total));
   LOGGER(INFO, "groupID:%d pid:%d GPU:%d memUsed:%ld MB before resumed", amem_groupID_value(), getpid(), dev_,
@@ -994,7 +1037,7 @@ int Engine::resume(Ctx& c, bool* incomplete) {
     note(e);
     if (e == hipSuccess) {
       note(h_sums_verify_.ensure(nch * sizeof(ChunkSum)));
-      note(CHECK_HIP(hipMemcpy(h_sums_verify_.p, d_sums_.p, nch * sizeof(ChunkSum), hipMemcpyDeviceToHost)));
+      note(CHECK_HIP(hipMemcpy(h_sums_verify_.p, d_sums_.p, nch * sizeof(ChunkSum), hipMemcpyDefault)));
       const ChunkSum* before = (const ChunkSum*)h_sums_.p;
       const ChunkSum* after = (const ChunkSum*)h_sums_verify_.p;
       uint64_t a = 0;

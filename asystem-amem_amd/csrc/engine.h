@@ -30,6 +30,7 @@ struct Options {
   int64_t hbm_wgs = 65536;                // workgroup cap of device-only kernels
   int64_t resume_batch_bytes = 64ll << 20;
   int64_t peer_timeout_ms = 60000;
+  int64_t scratch_on_host = 0;            // 1: engine tables live in pinned host memory even if the device has room
   int64_t pool_limit_bytes = 0;           // cap on pinned host memory a pause may need, 0 = none
   int64_t offload_free_tag = -1;          // caller tag whose regions are released without being copied
   int64_t peer_loopback = 0;              // let a process register with / update its own service (tests)
@@ -38,9 +39,11 @@ Options& options();
 
 // Growable device / pinned-host scratch.
 struct DevBuf {
-  void* p = nullptr;
+  void* p = nullptr;     // address the GPU uses
+  void* host = nullptr;  // set when the buffer lives in pinned host memory
   size_t cap = 0;
-  hipError_t ensure(size_t bytes);
+  // grow_on_host: if the buffer has to grow, put it in pinned host memory without trying the device
+  hipError_t ensure(size_t bytes, bool grow_on_host = false);
   void release();
 };
 struct PinBuf {
@@ -89,6 +92,7 @@ class Engine {
  private:
   hipError_t run_scan(const std::vector<ScanSeg>& segs, uint64_t* nchunks_out, bool want_sums,
                       float* ms);
+  hipError_t reserve_descs(size_t n);
   hipError_t upload_descs(const CopyDesc* descs, size_t n, uint64_t* ntiles_out);
   hipError_t upload_slab_table();
   hipError_t pause_copy_direct(Ctx& c, std::vector<Region*>& regs);
@@ -104,6 +108,7 @@ class Engine {
   hipStream_t dstream_ = nullptr;  // hipMemcpyAsync
   SlabPool* pool_ = nullptr;
   size_t slab_table_count_ = 0;
+  bool grow_on_host_ = false;  // set for the length of a resume
 
   DevBuf d_segs_, d_prefix_, d_flags_, d_sums_, d_descs_, d_tiles_, d_slabtab_;
   DevBuf d_staging_[2];

@@ -46,6 +46,8 @@ hipError_t launch_move(bool scatter, const CopyDesc* d_descs, const uint64_t* d_
                        const SlabTable& slabs, uint64_t off_base, uint32_t max_blocks, uint32_t xcds,
                        hipStream_t stream);
 
+// Makes the runtime load this library's device code now rather than at the first launch.
+hipError_t preload_kernels();
 hipError_t launch_calib_copy(const void* d_src, void* d_dst, uint64_t bytes, hipStream_t stream);
 
 }  // namespace amem

@@ -226,6 +226,17 @@ hipError_t launch_move(bool scatter, const CopyDesc* d_descs, const uint64_t* d_
   return hipGetLastError();
 }
 
+hipError_t preload_kernels() {
+  const void* fns[] = {(const void*)scan_chunks, (const void*)move_tiles<0>, (const void*)move_tiles<1>,
+                       (const void*)calib_copy};
+  for (const void* f : fns) {
+    hipFuncAttributes attr;
+    hipError_t e = hipFuncGetAttributes(&attr, f);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
 hipError_t launch_calib_copy(const void* d_src, void* d_dst, uint64_t bytes, hipStream_t stream) {
   const uint64_t nvec = bytes >> 4;
   if (nvec == 0) return hipSuccess;

@@ -19,7 +19,7 @@ GiB = 1 << 30
 @pytest.fixture()
 def eng(gpu, fresh):
     defaults = {k: fresh.amem_get_option(k) for k in (b"zero_elide", b"verify", b"pause_path", b"dma_min_bytes",
-                                                       b"staging_bytes", b"resume_batch_bytes")}
+                                                       b"staging_bytes", b"resume_batch_bytes", b"scratch_on_host")}
     yield fresh
     fresh.amem_mem_resume(0, 0)        # a test that failed mid-cycle must not leave the engine paused
     for k, v in defaults.items():
@@ -121,7 +121,7 @@ def test_repeated_cycles_with_writes_between(eng):
     regs.free()
 
 
-@pytest.mark.parametrize("opts", [{"zero_elide": 0}, {"pause_path": 0, "dma_min_bytes": 128 << 10},
+@pytest.mark.parametrize("opts", [{"zero_elide": 0}, {"scratch_on_host": 1}, {"scratch_on_host": 1, "pause_path": 1}, {"pause_path": 0, "dma_min_bytes": 128 << 10},
                                   {"staging_bytes": 8 << 20}, {"resume_batch_bytes": 1},
                                   {"staging_bytes": 1 << 20, "resume_batch_bytes": 1 << 40},
                                   {"pause_path": 3, "interleave_bytes": 1 << 16}, {"pause_path": 4}])
@@ -404,4 +404,38 @@ def test_config4_packed_granules_cycle(eng):
     assert st["local_regions"] == fp.ngranules and st["footprint_bytes"] == fp.total_bytes
     assert H.compare_tables(before, regs.table()) == []
     assert regs.mismatched_bytes() == 0
+    regs.free()
+
+
+def test_first_pause_on_a_full_device(eng):
+    """A process is usually paused because device memory is needed, so the first pause may find none
+    left for the engine's own tables. They then go to pinned host memory and the cycle is the same.
+    The device is filled from the host with plain allocations down to the last 64 KiB block."""
+    lib = eng
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+    hip.hipFree.argtypes = [C.c_void_p]
+    fp = Footprint(2, 19, max_regions=40, threads=8)
+    regs = H.Regions(lib, fp)
+    hogs = []
+
+    def grab(size, most):
+        for _ in range(most):
+            p = C.c_void_p()
+            if hip.hipMalloc(C.byref(p), size) != 0:
+                return
+            hogs.append(p)
+
+    grab(H.mem_free(lib) - 2 * GiB, 1)
+    grab(64 * MiB, 64); grab(2 * MiB, 64); grab(64 << 10, 256)
+    try:
+        free_full = H.mem_free(lib)
+        assert free_full < 64 * MiB
+        assert lib.amem_mem_pause(0, 0) == 0
+        assert H.mem_free(lib) - free_full > 0.9 * fp.total_bytes
+        assert lib.amem_mem_resume(0, 0) == 0
+        assert regs.mismatched_bytes() == 0
+    finally:
+        for p in hogs:
+            assert hip.hipFree(p) == 0
     regs.free()
