@@ -111,6 +111,7 @@ hipEvent_t Engine::event_at(size_t i) {
 }
 
 uint64_t Engine::trim_pool() {
+  std::lock_guard<std::mutex> busy(busy_);
   if (!pool_) return 0;
   slab_table_count_ = 0;
   return pool_->trim();
@@ -181,6 +182,7 @@ static bool inside_known_memory(uint64_t va, uint64_t bytes, uint64_t hint[2]) {
 
 hipError_t Engine::zero_scan(const amem_extent* ext, uint64_t n, uint8_t* flags, amem_chunk_sum* sums,
                              float* ms) {
+  std::lock_guard<std::mutex> busy(busy_);
   hipError_t e = init();
   if (e != hipSuccess) return e;
   std::vector<ScanSeg> segs(n);
@@ -293,6 +295,7 @@ static void emit_runs(const uint8_t* flags, uint64_t va, uint64_t size, bool eli
 
 hipError_t Engine::move(bool scatter, const amem_copy_desc* descs, uint64_t n, void* staging,
                         uint64_t staging_bytes, bool host_side, float* ms) {
+  std::lock_guard<std::mutex> busy(busy_);
   hipError_t e = init();
   if (e != hipSuccess) return e;
   if (ms) *ms = 0;
@@ -663,6 +666,7 @@ hipError_t Engine::pause_copy_staged(Ctx& c, std::vector<Region*>& regs, bool* u
 }
 
 int Engine::pause(Ctx& c, bool* rolled_back) {
+  std::lock_guard<std::mutex> busy(busy_);
   auto t0 = Clock::now();
   if (rolled_back) *rolled_back = false;
   hipError_t e = init();
@@ -883,6 +887,7 @@ void Engine::forget(uint64_t va) {
 // ---------------------------------------------------------------------------------------
 
 int Engine::resume(Ctx& c, bool* incomplete) {
+  std::lock_guard<std::mutex> busy(busy_);
   if (incomplete) *incomplete = false;
   hipError_t e = init();
   if (e != hipSuccess) return (int)e;
@@ -1125,6 +1130,7 @@ int Engine::resume(Ctx& c, bool* incomplete) {
 // ---------------------------------------------------------------------------------------
 
 hipError_t Engine::probe_link(uint64_t bytes, int reps, double* d2h, double* h2d) {
+  std::lock_guard<std::mutex> busy(busy_);
   hipError_t e = init();
   if (e != hipSuccess) return e;
   void *hp = nullptr, *dp = nullptr;
@@ -1153,6 +1159,7 @@ hipError_t Engine::probe_link(uint64_t bytes, int reps, double* d2h, double* h2d
 }
 
 hipError_t Engine::calib_copy(uint64_t bytes, int reps, float* ms) {
+  std::lock_guard<std::mutex> busy(busy_);
   hipError_t e = init();
   if (e != hipSuccess) return e;
   bytes &= ~(uint64_t)15;

@@ -8,6 +8,7 @@
 #include <hip/hip_runtime_api.h>
 #include <stdint.h>
 
+#include <mutex>
 #include <vector>
 
 #include "ctx.h"
@@ -103,6 +104,9 @@ class Engine {
   hipEvent_t event_at(size_t i);
 
   int dev_;
+  // One caller at a time: every entry point uses the same scratch tables and streams.
+  // Taken after Ctx::structure where both are held.
+  std::mutex busy_;
   bool inited_ = false;
   hipStream_t kstream_ = nullptr;  // kernels
   hipStream_t dstream_ = nullptr;  // hipMemcpyAsync

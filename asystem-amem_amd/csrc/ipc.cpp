@@ -1,3 +1,6 @@
+#ifndef _GNU_SOURCE
+#define _GNU_SOURCE 1
+#endif
 #include "ipc.h"
 
 #include <errno.h>
@@ -157,8 +160,22 @@ void serve() {
     if (n < 0) { if (errno == EINTR) continue; break; }
     if (fds[1].revents) break;
     if (fds[0].revents & POLLIN) {
-      int c = accept(g_svc.listen_fd, nullptr, nullptr);
-      if (c >= 0) fds.push_back({c, POLLIN, 0});
+      int c = accept4(g_svc.listen_fd, nullptr, nullptr, SOCK_CLOEXEC);
+      if (c >= 0) {
+        // Requests change this process's address space: only this user's processes may send
+        // them, and one that stops half-way through a message must not block the others.
+        struct ucred cred = {};
+        socklen_t len = sizeof(cred);
+        if (getsockopt(c, SOL_SOCKET, SO_PEERCRED, &cred, &len) != 0 || cred.uid != geteuid()) {
+          LOGGER(WARN, "pid:%d refused a connection from uid %d", getpid(), (int)cred.uid);
+          close(c);
+        } else {
+          struct timeval tv = {5, 0};
+          setsockopt(c, SOL_SOCKET, SO_RCVTIMEO, &tv, sizeof(tv));
+          setsockopt(c, SOL_SOCKET, SO_SNDTIMEO, &tv, sizeof(tv));
+          fds.push_back({c, POLLIN, 0});
+        }
+      }
     }
     for (size_t i = 2; i < fds.size();) {
       if (!(fds[i].revents & (POLLIN | POLLHUP | POLLERR))) { ++i; continue; }
@@ -182,13 +199,22 @@ void serve() {
 
 bool claim(int slot) {
   std::string lp = lock_name(slot);
-  int fd = open(lp.c_str(), O_CREAT | O_RDWR | O_CLOEXEC, 0666);
-  if (fd < 0) return false;
-  if (flock(fd, LOCK_EX | LOCK_NB) != 0) { close(fd); return false; }
-  g_svc.lock_fd = fd;
-  g_svc.lock_path = lp;
-  g_svc.slot = slot;
-  return true;
+  for (int attempt = 0; attempt < 4; ++attempt) {
+    int fd = open(lp.c_str(), O_CREAT | O_RDWR | O_CLOEXEC, 0666);
+    if (fd < 0) return false;
+    if (flock(fd, LOCK_EX | LOCK_NB) != 0) { close(fd); return false; }
+    // The lock is on the file, not on its name: if the name was removed or replaced between the
+    // open and the lock (a /tmp cleaner), somebody else may hold a lock under the same name.
+    struct stat a, b;
+    if (fstat(fd, &a) == 0 && stat(lp.c_str(), &b) == 0 && a.st_ino == b.st_ino && a.st_dev == b.st_dev) {
+      g_svc.lock_fd = fd;
+      g_svc.lock_path = lp;
+      g_svc.slot = slot;
+      return true;
+    }
+    close(fd);
+  }
+  return false;
 }
 
 // Connect to the service of `slot`, waiting for it to appear (connect_if_not,
@@ -300,7 +326,8 @@ void ipc_stop() {
     if (g_svc.conn[i] >= 0) close(g_svc.conn[i]);
     g_svc.conn[i] = -1;
   }
-  unlink(g_svc.lock_path.c_str());
+  // The lock file stays: removing the name while another process is between open() and flock()
+  // on it would let two processes hold "the" lock of one slot.
   close(g_svc.lock_fd);
   g_svc.lock_fd = g_svc.listen_fd = -1;
   g_svc.slot = -1;

@@ -134,7 +134,17 @@ hipError_t vmm_create_map(uint64_t va, int dev, size_t size, uint64_t* new_handl
   hipError_t e = CHECK_HIP(hipMemCreate(&h, size, &prop, 0));
   if (e != hipSuccess) return e;
   e = CHECK_HIP(hipMemMap((void*)(uintptr_t)va, size, 0, h, 0));
-  if (e == hipSuccess) e = CHECK_HIP(set_rw(va, size, dev));
+  if (e == hipSuccess) {
+    e = CHECK_HIP(set_rw(va, size, dev));
+    if (e != hipSuccess) (void)hipMemUnmap((void*)(uintptr_t)va, size);
+  }
+  if (e != hipSuccess) {
+    // leave the address as it was found: reserved, nothing mapped, no memory held
+    (void)hipMemRelease(h);
+    (void)hipGetLastError();
+    *new_handle = 0;
+    return e;
+  }
   *new_handle = handle_bits(h);
   return e;
 }
@@ -154,14 +164,25 @@ hipError_t vmm_import_map(int dev, uint64_t va, size_t size, int fd, bool close_
                                                            hipMemHandleTypePosixFileDescriptor));
   if (e == hipSuccess) {
     e = CHECK_HIP(hipMemMap((void*)(uintptr_t)va, size, 0, h, 0));
-    if (e == hipSuccess) e = CHECK_HIP(set_rw(va, size, dev));
-    else LOGGER(ERROR, "pid:%d newMap ret:%d", getpid(), (int)e);
+    if (e == hipSuccess) {
+      e = CHECK_HIP(set_rw(va, size, dev));
+      if (e != hipSuccess) (void)hipMemUnmap((void*)(uintptr_t)va, size);
+    } else {
+      LOGGER(ERROR, "pid:%d newMap ret:%d", getpid(), (int)e);
+    }
+    if (e != hipSuccess) {
+      LOGGER(ERROR, "pid:%d curDev:%d newHandle:%llx inFD:%d ret:%d", getpid(), dev,
+             (unsigned long long)handle_bits(h), fd, (int)e);
+      (void)hipMemRelease(h);  // the import's reference; nothing is mapped
+      (void)hipGetLastError();
+      h = nullptr;
+    }
+  } else {
+    LOGGER(ERROR, "pid:%d curDev:%d import of inFD:%d ret:%d", getpid(), dev, fd, (int)e);
+    h = nullptr;
   }
   if (close_fd) close(fd);
   if (new_handle) *new_handle = handle_bits(h);
-  if (e != hipSuccess)
-    LOGGER(ERROR, "pid:%d curDev:%d newHandle:%llx inFD:%d ret:%d", getpid(), dev,
-           (unsigned long long)handle_bits(h), fd, (int)e);
   return e;
 }
 
