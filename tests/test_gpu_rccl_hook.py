@@ -76,3 +76,82 @@ def test_hook_registers_and_releases_rccl_style_allocations(gpu, tmp_path):
     env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="1", AMEM_IPC="0")
     r = subprocess.run([sys.executable, "-c", CHILD, ROOT, standin], env=env, capture_output=True, text=True, timeout=240)
     assert r.returncode == 0 and "rccl hook ok" in r.stdout, (r.returncode, r.stdout[-3000:], r.stderr[-3000:])
+
+
+REAL_RCCL_CHILD = r'''
+import ctypes as C, os, sys
+import numpy as np
+root = sys.argv[1]
+sys.path.insert(0, root)
+libdir = os.path.join(root, "asystem-amem_amd", "lib")
+hook = C.CDLL(os.path.join(libdir, "libamem_rccl_hook.so"), mode=C.RTLD_GLOBAL)   # before the runtime and RCCL
+from asystem_amem_amd import binding as B, harness as H
+lib = B.load()
+hip = C.CDLL("libamdhip64.so")
+try:
+    rccl = C.CDLL("librccl.so")
+except OSError as e:
+    print("no librccl.so:", e); print("rccl skipped"); sys.exit(0)
+hook.amem_rccl_hook_registered.restype = C.c_int64
+class UID(C.Structure):
+    _fields_ = [("b", C.c_char * 128)]
+rccl.ncclCommInitRank.argtypes = [C.POINTER(C.c_void_p), C.c_int, UID, C.c_int]
+rccl.ncclAllReduce.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+rccl.ncclCommDestroy.argtypes = [C.c_void_p]
+assert hip.hipSetDevice(0) == 0
+uid, comm = UID(), C.c_void_p()
+assert rccl.ncclGetUniqueId(C.byref(uid)) == 0
+assert rccl.ncclCommInitRank(C.byref(comm), 1, uid, 0) == 0
+# the buffers of the collective: tracked VMM memory, the way the reference's nccl-tests patch
+# allocates them with ncclMemAlloc
+MiB = 1 << 20
+n = 4 * MiB // 4
+bufs = []
+for _ in range(2):
+    va, h, asz = C.c_uint64(), C.c_uint64(), C.c_uint64()
+    assert lib.amem_vmm_alloc(4 * MiB, 0, C.byref(va), C.byref(h), C.byref(asz)) == 0
+    assert lib.amem_add_alloc_info(va.value, asz.value, B.TYPE_LOCAL, 0, h.value, -1, 0, None, B.CALLER_P2P) == 0
+    bufs.append((va.value, asz.value))
+send, recv = bufs[0][0], bufs[1][0]
+rng = np.random.default_rng(5)
+
+def allreduce_wrong():
+    x = rng.standard_normal(n).astype(np.float32)
+    assert lib.amem_copy_to_device(send, x.ctypes.data, x.nbytes) == 0
+    junk = np.full(n, -1.0, dtype=np.float32)
+    assert lib.amem_copy_to_device(recv, junk.ctypes.data, junk.nbytes) == 0
+    assert rccl.ncclAllReduce(send, recv, n, 7, 0, comm, None) == 0            # ncclFloat32, ncclSum, null stream
+    assert hip.hipDeviceSynchronize() == 0
+    y = np.empty_like(x)
+    assert lib.amem_copy_from_device(y.ctypes.data, recv, y.nbytes) == 0
+    return int(np.count_nonzero(x != y))                                        # one rank: the sum is the input
+
+assert allreduce_wrong() == 0
+by_hook = hook.amem_rccl_hook_registered()
+print("regions RCCL allocated through the VMM API:", by_hook)
+assert lib.amem_region_count(0) == 2 + by_hook
+for cycle in range(3):
+    free0 = H.mem_free(lib)
+    assert lib.ncclPause(None) == 0 and lib.amem_check_paused(0) == 1
+    assert H.mem_free(lib) - free0 >= 6 * MiB
+    assert lib.ncclResume(None) == 0 and lib.amem_check_paused(0) == 0
+    assert allreduce_wrong() == 0, cycle                                       # same addresses, same communicator
+assert rccl.ncclCommDestroy(comm) == 0
+for va, asz in bufs:
+    assert lib.amem_del_alloc_info(va, 0, 0) == 0 and lib.amem_vmm_free(va, asz, 0) == 0
+assert lib.amem_region_count(0) == hook.amem_rccl_hook_registered()
+print("rccl ok")
+'''
+
+
+def test_real_rccl_communicator_works_across_cycles(gpu):
+    """The check the reference puts into nccl-tests (nccl_patch/nccl-tests.diff:24-50: pause and
+    resume between iterations, then #wrong must be 0), on a one-rank communicator of the RCCL that
+    ships with ROCm, with the hook library in place: an all-reduce between tracked buffers gives
+    the right answer before a cycle and after each of three."""
+    env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="1", AMEM_IPC="0", NCCL_CUMEM_ENABLE="1")
+    r = subprocess.run([sys.executable, "-c", REAL_RCCL_CHILD, ROOT], env=env, capture_output=True, text=True, timeout=240)
+    assert r.returncode == 0 and ("rccl ok" in r.stdout or "rccl skipped" in r.stdout), \
+        (r.returncode, r.stdout[-3000:], r.stderr[-3000:])
+    if "rccl skipped" in r.stdout:
+        pytest.skip("librccl.so is not loadable on this machine")
