@@ -144,6 +144,7 @@ int amem_add_alloc_info(uint64_t va, uint64_t size, int type, int dev, uint64_t 
       r.mcHandle = peer_handle;  // the ctor's in_mcHandle slot receives peerHandle (amem_nccl.cpp:145)
       r.oosFlag = oosFlag;
       r.handleGen = 1;
+      if (peerFlag) r.ownerSlot = peer_dev;
       table.emplace(va, r);
       if (caller >= 0 && caller < AMEM_MAX_CALLER) c->allocBytes[caller] += size;
       if (peerFlag && gpu_present()) srcDevDetected = vmm_handle_device(handle);
@@ -194,6 +195,11 @@ int amem_add_alloc_info(uint64_t va, uint64_t size, int type, int dev, uint64_t 
     // holds the slot equal to its device ordinal; with several processes on one GPU (the
     // owner's device is then this process's own device) the owner cannot be told apart.
     if (srcDevDetected >= 0 && srcDevDetected != dev) {
+      {
+        std::lock_guard<std::mutex> lf(c->fields);
+        auto it = c->allocTable[dev].find(va);
+        if (it != c->allocTable[dev].end()) it->second.ownerSlot = srcDevDetected;
+      }
       ret = peer_register(peer_handle, va, srcDevDetected);
       if (ret != 0) {
         LOGGER(WARN, "ALLocInfo: communication failed. groupID:%d pid:%d allocSz:%ld curDev:%d dptr:%llx "

@@ -40,6 +40,7 @@ struct Region {
   // engine bookkeeping (no reference counterpart)
   uint64_t parkedBytes = 0;
   uint64_t handleGen = 0;
+  int ownerSlot = -1;  // imported regions: slot of the owning process, when known
 };
 
 static inline bool from_peer(int type) { return type > AMEM_TYPE_LOCAL_SYMM; }  // amem_nccl.h:82-84

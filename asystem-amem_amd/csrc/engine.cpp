@@ -1092,14 +1092,33 @@ int Engine::resume(Ctx& c, bool* incomplete) {
     std::unique_lock<std::mutex> lk(c.fields);
     const int64_t tmo = options().peer_timeout_ms;
     auto done = [&] { return c.releaseShadowCnt <= 0; };
-    if (tmo > 0) {
-      if (!c.shadow_cv.wait_for(lk, std::chrono::milliseconds(tmo), done)) {
+    // True when every import still waiting belongs to a process that no longer exists.
+    auto owners_gone = [&] {
+      bool any = false;
+      for (auto& kv : table) {
+        const Region& r = kv.second;
+        if (!from_peer(r.type) || r.state != AMEM_STATE_HOLE) continue;
+        any = true;
+        if (r.ownerSlot < 0 || peer_alive(r.ownerSlot)) return false;
+      }
+      return any;
+    };
+    const auto t_wait = Clock::now();
+    while (!done()) {
+      c.shadow_cv.wait_for(lk, std::chrono::milliseconds(200), done);
+      if (done()) break;
+      if (owners_gone()) {
+        LOGGER(ERROR, "groupID:%d pid:%d GPU:%d peerLeft:%d and their owners are gone, giving up",
+               amem_groupID_value(), getpid(), dev_, c.releaseShadowCnt);
+        if (rc == 0) rc = 1;
+        break;
+      }
+      if (tmo > 0 && ms_since(t_wait) >= (double)tmo) {
         LOGGER(ERROR, "groupID:%d pid:%d GPU:%d peerLeft:%d after %lld ms, giving up", amem_groupID_value(),
                getpid(), dev_, c.releaseShadowCnt, (long long)tmo);
         if (rc == 0) rc = 1;
+        break;
       }
-    } else {
-      c.shadow_cv.wait(lk, done);
     }
   }
   stats_.resume_peer_ms = ms_since(tpeer);

@@ -217,6 +217,17 @@ bool claim(int slot) {
   return false;
 }
 
+// True while some process holds the lock file of `slot`. The lock dies with its holder, so
+// this is how a peer that crashed is told from one that is merely slow.
+bool slot_claimed(int slot) {
+  int fd = open(lock_name(slot).c_str(), O_RDWR | O_CLOEXEC);
+  if (fd < 0) return false;
+  const bool held = flock(fd, LOCK_SH | LOCK_NB) != 0;
+  if (!held) flock(fd, LOCK_UN);
+  close(fd);
+  return held;
+}
+
 // Connect to the service of `slot`, waiting for it to appear (connect_if_not,
 // gmm_client_impl.cpp:288-347, with a bounded wait instead of an abort).
 int connect_if_not(int slot) {
@@ -239,6 +250,13 @@ int connect_if_not(int slot) {
       return s;
     }
     close(s);
+    // A peer is known by its slot only after it has claimed that slot, so an unclaimed slot
+    // means its process is gone; a claimed one without a socket yet is still starting.
+    if (!slot_claimed(slot)) {
+      LOGGER(ERROR, "groupID:%d pid:%d the process of slot %d is gone (nobody holds %s)", amem_groupID_value(),
+             getpid(), slot, lock_name(slot).c_str());
+      return -1;
+    }
     if (waited >= budget_ms) break;
     usleep(20000);
   }
@@ -268,6 +286,8 @@ int rpc(int slot, const WireReq& req, int fd) {
 }  // namespace
 
 int ipc_slot() { return g_svc.slot; }
+
+bool peer_alive(int slot) { return slot >= 0 && slot < AMEM_MAX_DEVS && slot_claimed(slot); }
 
 int ipc_start(int preferred) {
   std::lock_guard<std::mutex> lk(g_svc.mtx);

@@ -20,6 +20,8 @@ int amem_groupID_value();
 int ipc_start(int preferred);
 void ipc_stop();
 int ipc_slot();
+// Whether a process currently holds `slot` of this group (a crashed one no longer does).
+bool peer_alive(int slot);
 
 // Importer -> owner: "my VA `my_va` maps your handle `src_handle`".
 // 0 ok; 1 when the owner is this process (the reference's is_sameProcess rule,

@@ -70,3 +70,51 @@ def test_register_peer_across_processes():
         owner.join(30)
         assert imp.exitcode == 0 and owner.exitcode == 0
         assert not [f for f in os.listdir(ipc_dir) if f.endswith(".sock")]   # sockets removed on shutdown
+
+
+def _late_importer(ipc_dir, gid, owner_slot, to_parent, from_parent):
+    import time
+    os.environ.update(AMEM_ENABLE="1", GMM_LOG="1", GMM_IPC_DIR=ipc_dir, AMEM_GROUPID=str(gid))
+    from asystem_amem_amd import binding as B
+    lib = B.load()
+    lib.amem_set_option(b"peer_timeout_ms", 30000)
+    my_va = 0x7f3000000000
+    first = lib.amem_add_alloc_info(my_va, 4 * MiB, B.TYPE_PEER_POSIX, 0, 0x211, owner_slot, OWNER_HANDLE, None,
+                                    B.CALLER_P2P_PEER)
+    to_parent.send(("first", first))
+    assert from_parent.recv() == "owner is dead"
+    t0 = time.perf_counter()
+    second = lib.amem_add_alloc_info(my_va + (1 << 30), 4 * MiB, B.TYPE_PEER_POSIX, 0, 0x212, owner_slot, OWNER_HANDLE,
+                                     None, B.CALLER_P2P_PEER)
+    # the first failure dropped the connection; this one has to find out from the stale socket file
+    third = lib.amem_add_alloc_info(my_va + (2 << 30), 4 * MiB, B.TYPE_PEER_POSIX, 0, 0x213, owner_slot, OWNER_HANDLE,
+                                    None, B.CALLER_P2P_PEER)
+    to_parent.send(("second", second, third, time.perf_counter() - t0))
+    assert from_parent.recv() == "exit"
+    lib.amem_shutdown()
+
+
+def test_a_peer_that_died_is_noticed_at_once():
+    """Failure detection the reference lacks (its connect loop retries for a fixed time and then aborts the
+    process, gmm_client_impl.cpp:288-347): a slot's lock dies with its holder, so a request to a peer
+    whose process was killed fails within a moment instead of waiting out the 30 s timeout."""
+    ctx = mp.get_context("spawn")
+    with tempfile.TemporaryDirectory() as ipc_dir:
+        gid = 0x6000 + os.getpid() % 4096
+        o_out, o_in = ctx.Pipe(), ctx.Pipe()
+        owner = ctx.Process(target=_owner, args=(ipc_dir, gid, o_out[1], o_in[0]))
+        owner.start()
+        tag, owner_slot = o_out[0].recv()
+        i_out, i_in = ctx.Pipe(), ctx.Pipe()
+        imp = ctx.Process(target=_late_importer, args=(ipc_dir, gid, owner_slot, i_out[1], i_in[0]))
+        imp.start()
+        assert i_out[0].poll(60) and i_out[0].recv() == ("first", 0)
+        owner.kill()                                       # this very process, by its pid; no clean-up runs
+        owner.join(30)
+        i_in[1].send("owner is dead")
+        assert i_out[0].poll(60)
+        tag, second, third, seconds = i_out[0].recv()
+        assert tag == "second" and second == 1 and third == 1 and seconds < 2.0
+        i_in[1].send("exit")
+        imp.join(30)
+        assert imp.exitcode == 0
