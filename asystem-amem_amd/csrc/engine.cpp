@@ -1073,7 +1073,16 @@ int Engine::resume(Ctx& c, bool* incomplete) {
     for (int s = 0; s < AMEM_MAX_DEVS; ++s) {
       if (peers[s] == 0) continue;
       int ret = peer_update(s, peers[s], x.fd);
-      if (ret != 0) {
+      if (ret != 0 && !peer_alive(s)) {
+        // The importer's process is gone and its mapping with it: nothing to update, now or later.
+        LOGGER(WARN, "groupID:%d pid:%d localDptr:%llx the importer in slot %d is gone, forgetting its mapping %llx",
+               amem_groupID_value(), getpid(), (unsigned long long)x.va, s, (unsigned long long)peers[s]);
+        std::lock_guard<std::mutex> lk(c.fields);
+        x.r->peers[s] = 0;
+        x.r->hasPeer = false;
+        for (int k = 0; k < AMEM_MAX_DEVS; ++k) x.r->hasPeer |= x.r->peers[k] != 0;
+        c.releaseLocalCnt--;
+      } else if (ret != 0) {
         LOGGER(ERROR, "groupID:%d pid:%d localDptr:%llx newHandle:%llx fd:%d notify peer %d to remap dptr:%llx ret:%d",
                amem_groupID_value(), getpid(), (unsigned long long)x.va, (unsigned long long)x.r->handle, x.fd,
                s, (unsigned long long)peers[s], ret);

@@ -332,3 +332,28 @@ def test_importer_times_out_when_owner_never_re_exports(gpu, fresh):
         lib.amem_mem_resume(0, 0)
         lib.amem_set_option(b"peer_loopback", 0)
         lib.amem_set_option(b"peer_timeout_ms", old_to)
+
+
+def test_owner_forgets_an_importer_whose_process_is_gone(gpu, fresh):
+    """An owner holds the address of an importer in a slot nobody holds (its process died). Resume
+    finds that out from the slot's lock, drops the stale entry and succeeds; the next cycle no
+    longer tries. Nothing is killed here: the slot simply never had a holder."""
+    from asystem_amem_amd import binding as B, harness as H
+    from asystem_amem_amd.footprint import Footprint
+    lib = fresh
+    fp = Footprint(2, 14, max_regions=3, threads=2)
+    regs = H.Regions(lib, fp)
+    ghost = (lib.amem_get_slot() + 3) % 8
+    assert lib.amem_add_peer_info(int(regs.va[1]), 0x7f5500000000, ghost) == 0
+    assert H.region_table(lib, 0)[int(regs.va[1])]["has_peer"] == 1
+    assert lib.amem_mem_pause(0, 0) == 0
+    assert H.counters(lib)["release_local_cnt"] == 1
+    t0 = time.perf_counter()
+    assert lib.amem_mem_resume(0, 0) == 0
+    assert time.perf_counter() - t0 < 5.0                      # no waiting for a peer that cannot answer
+    r = H.region_table(lib, 0)[int(regs.va[1])]
+    assert r["has_peer"] == 0 and not any(r["peers"]) and H.counters(lib)["release_local_cnt"] == 0
+    assert regs.mismatched_bytes() == 0
+    assert lib.amem_mem_pause(0, 0) == 0 and H.counters(lib)["release_local_cnt"] == 0
+    assert lib.amem_mem_resume(0, 0) == 0 and regs.mismatched_bytes() == 0
+    regs.free()
