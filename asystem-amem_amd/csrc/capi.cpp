@@ -607,6 +607,7 @@ static OptRef* opt_table(size_t* n) {
       {"offload_free_tag", &o.offload_free_tag, -1, AMEM_MAX_CALLER - 1},
       {"pool_limit_bytes", &o.pool_limit_bytes, 0, (int64_t)1 << 46},
       {"scratch_on_host", &o.scratch_on_host, 0, 1},
+      {"release_thread", &o.release_thread, 0, 1},
   };
   *n = sizeof(t) / sizeof(t[0]);
   return t;

@@ -356,7 +356,7 @@ static int popcount_peers(const Region& r) {
 
 // Reference step 3 for one region (amem_nccl.cpp:529-557): drop the mapping and every
 // reference, mark HOLE, forget the handle.
-hipError_t Engine::release_local(Ctx& c, Region* r, uint64_t va) {
+hipError_t Engine::release_local(Ctx& c, Region* r, uint64_t va, std::pair<uint64_t, int>* deferred) {
   auto t0 = Clock::now();
   uint64_t old = r->handle ? r->handle : vmm_handle_of(va);
   if (r->type == AMEM_TYPE_LOCAL_SYMM)
@@ -365,7 +365,13 @@ hipError_t Engine::release_local(Ctx& c, Region* r, uint64_t va) {
   if (r->refcount > 0)
     LOGGER(DEBUG, "memPause: groupID:%d pid:%d dptr:%llx refcount:%d", amem_groupID_value(), getpid(),
            (unsigned long long)va, r->refcount);
-  hipError_t e = vmm_unmap_release(va, r->allocSz, old, r->refcount);
+  hipError_t e;
+  if (deferred) {
+    e = vmm_unmap(va, r->allocSz);
+    *deferred = {old, r->refcount};
+  } else {
+    e = vmm_unmap_release(va, r->allocSz, old, r->refcount);
+  }
   {
     std::lock_guard<std::mutex> lk(c.fields);
     c.releaseLocalCnt += popcount_peers(*r);
@@ -456,9 +462,9 @@ hipError_t Engine::pause_copy_direct(Ctx& c, std::vector<Region*>& regs) {
 struct PauseShape { uint32_t wgs, xcds; double gbps, unmap_ms; };
 static PauseShape choose_pause_shape(uint64_t parked_bytes, size_t regions) {
   static const PauseShape shapes[] = {
-      {4, 1, 44.0, 0.29},   // 4 workgroups on one XCD
-      {8, 1, 47.0, 0.32},
-      {32, 1, 50.0, 0.42},  // one XCD, saturated
+      {4, 1, 44.0, 0.28},   // 4 workgroups on one XCD
+      {8, 1, 50.0, 0.28},
+      {32, 1, 52.0, 0.30},  // one XCD, saturated
       {96, 8, 56.0, 2.0},   // the whole chip: fastest copy, unmaps crawl while it runs
   };
   const double idle_unmap_ms = 0.26;
@@ -475,8 +481,10 @@ static PauseShape choose_pause_shape(uint64_t parked_bytes, size_t regions) {
 
 // Interleaved path: the gather kernel writes pinned host memory itself, in many short
 // launches (one per group of regions holding about interleave_bytes of parked data), with an
-// event after each. A second host thread unmaps and releases a group's regions as soon as
-// that group's event has fired. An unmap issued while kernels are queued waits for roughly
+// event after each. A second host thread unmaps a group's regions as soon as that group's
+// event has fired, and a third releases the handles behind it: the unmaps are what the pause
+// waits for at the end, so nothing else rides on their thread (release_thread = 0 puts the
+// releases back on it). An unmap issued while kernels are queued waits for roughly
 // one kernel boundary, and the kernels keep running at link rate meanwhile, so short
 // launches let most of the unmap time hide behind the transfer; a copy-engine transfer
 // would instead stall for the whole of every unmap.
@@ -506,20 +514,42 @@ hipError_t Engine::pause_copy_interleaved(Ctx& c, std::vector<Region*>& regs) {
   hipEvent_t start = event_at(ev0 + groups.size());  // creates every event before the thread starts
   std::atomic<size_t> launched{0};
   std::atomic<int> failed{0};
+  const bool split = options().release_thread != 0;
+  std::vector<std::pair<uint64_t, int>> to_release(split ? n : 0);
+  std::atomic<size_t> unmapped{0};
+  std::atomic<bool> unmapper_done{false};
   auto tc = Clock::now();
   std::thread unmapper([&] {
     (void)hipSetDevice(dev_);
     for (size_t g = 0; g < groups.size(); ++g) {
       while (launched.load(std::memory_order_acquire) <= g) {
-        if (failed.load()) return;
+        if (failed.load()) { unmapper_done.store(true); return; }
         std::this_thread::yield();
       }
       hipError_t es2 = CHECK_HIP(hipEventSynchronize(events_[ev0 + g]));
-      if (es2 != hipSuccess) { failed.store((int)es2); return; }
+      if (es2 != hipSuccess) { failed.store((int)es2); break; }
       for (size_t r = groups[g].r0; r < groups[g].r1; ++r) {
-        hipError_t e2 = release_local(c, regs[r], parked_[r].va);
-        if (e2 != hipSuccess) { failed.store((int)e2); return; }
+        hipError_t e2 = release_local(c, regs[r], parked_[r].va, split ? &to_release[r] : nullptr);
+        if (split) unmapped.store(r + 1, std::memory_order_release);
+        if (e2 != hipSuccess) { failed.store((int)e2); break; }
       }
+      if (failed.load()) break;
+    }
+    unmapper_done.store(true, std::memory_order_release);
+  });
+  std::thread releaser;
+  if (split) releaser = std::thread([&] {
+    (void)hipSetDevice(dev_);
+    size_t done = 0;
+    for (;;) {
+      const bool last = unmapper_done.load(std::memory_order_acquire);
+      const size_t avail = unmapped.load(std::memory_order_acquire);
+      for (; done < avail; ++done) {
+        hipError_t e2 = vmm_release(to_release[done].first, to_release[done].second);
+        if (e2 != hipSuccess && !failed.load()) failed.store((int)e2);
+      }
+      if (last && done == unmapped.load(std::memory_order_acquire)) break;
+      std::this_thread::yield();
     }
   });
   (void)CHECK_HIP(hipEventRecord(start, kstream_));
@@ -540,6 +570,7 @@ hipError_t Engine::pause_copy_interleaved(Ctx& c, std::vector<Region*>& regs) {
   }
   if (e != hipSuccess) failed.store((int)e);
   unmapper.join();
+  if (releaser.joinable()) releaser.join();
   hipError_t es = CHECK_HIP(hipStreamSynchronize(kstream_));
   stats_.pause_copy_ms = ms_since(tc);
   if (!groups.empty()) {

@@ -9,6 +9,7 @@
 #include <stdint.h>
 
 #include <mutex>
+#include <utility>
 #include <vector>
 
 #include "ctx.h"
@@ -31,6 +32,7 @@ struct Options {
   int64_t hbm_wgs = 65536;                // workgroup cap of device-only kernels
   int64_t resume_batch_bytes = 64ll << 20;
   int64_t peer_timeout_ms = 60000;
+  int64_t release_thread = 1;             // interleaved path: handles are released on a third thread
   int64_t scratch_on_host = 0;            // 1: engine tables live in pinned host memory even if the device has room
   int64_t pool_limit_bytes = 0;           // cap on pinned host memory a pause may need, 0 = none
   int64_t offload_free_tag = -1;          // caller tag whose regions are released without being copied
@@ -100,7 +102,8 @@ class Engine {
   hipError_t pause_copy_staged(Ctx& c, std::vector<Region*>& regs, bool* used);
   hipError_t pause_copy_interleaved(Ctx& c, std::vector<Region*>& regs);
   hipError_t pause_copy_reference(Ctx& c, std::vector<Region*>& regs);
-  hipError_t release_local(Ctx& c, Region* r, uint64_t va);
+  // With `deferred`, the mapping is removed but the handle is handed back to be released later.
+  hipError_t release_local(Ctx& c, Region* r, uint64_t va, std::pair<uint64_t, int>* deferred = nullptr);
   hipEvent_t event_at(size_t i);
 
   int dev_;

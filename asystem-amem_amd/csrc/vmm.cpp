@@ -128,6 +128,21 @@ hipError_t vmm_unmap_release(uint64_t va, size_t size, uint64_t handle, int extr
   return e;
 }
 
+hipError_t vmm_unmap(uint64_t va, size_t size) {
+  if (va == 0) return hipSuccess;
+  return CHECK_HIP(hipMemUnmap((void*)(uintptr_t)va, mapped_size(va, size)));
+}
+
+hipError_t vmm_release(uint64_t handle, int extra) {
+  hipError_t e = hipSuccess;
+  if (handle == 0) return e;
+  for (int k = 0; k <= (extra > 0 ? extra : 0); ++k) {
+    hipError_t e2 = CHECK_HIP(hipMemRelease(as_handle(handle)));
+    if (e == hipSuccess) e = e2;
+  }
+  return e;
+}
+
 hipError_t vmm_create_map(uint64_t va, int dev, size_t size, uint64_t* new_handle) {
   hipMemAllocationProp prop = device_prop(dev);
   hipMemGenericAllocationHandle_t h = nullptr;

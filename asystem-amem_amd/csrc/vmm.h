@@ -33,6 +33,9 @@ hipError_t vmm_free(uint64_t va, size_t alloc_size, uint64_t handle);
 // creator plus `extra` more (amem_cuMemReleaseHandle, amem_nccl.h:141-161, without its
 // retain/release pair: the registry already knows the handle).
 hipError_t vmm_unmap_release(uint64_t va, size_t size, uint64_t handle, int extra);
+// The two halves of vmm_unmap_release, for callers that run them on different threads.
+hipError_t vmm_unmap(uint64_t va, size_t size);
+hipError_t vmm_release(uint64_t handle, int extra);
 
 // New physical memory at an existing reservation (amem_cuAllocAndExport, amem_nccl.h:164-193).
 hipError_t vmm_create_map(uint64_t va, int dev, size_t size, uint64_t* new_handle);

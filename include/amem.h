@@ -282,6 +282,8 @@ int amem_set_enabled(int on);
  *                     AMEM_NCCL_OFFLOAD_FREE_TAG is documented to do in the reference, where the
  *                     variable is parsed but never takes effect (amem_nccl.cpp:40, :503, :620);
  *                     the environment variable stays ineffective here too, only this option acts
+ *   "release_thread"  0/1 (default 1): the default pause path releases handles on a thread of their own
+ *                     instead of on the one that unmaps
  *   "scratch_on_host" 0/1: keep the engine's own tables in pinned host memory. That is where they go
  *                     anyway when the device has no room for them at pause time; 1 forces it
  *   "pool_limit_bytes" most pinned host memory one pause may need (0 = no limit). A pause that
