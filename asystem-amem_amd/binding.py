@@ -108,6 +108,7 @@ _SIGNATURES = {
     "amem_set_option": (C.c_int, [C.c_char_p, C.c_int64]),
     "amem_get_option": (C.c_int64, [C.c_char_p]),
     "amem_pool_trim": (C.c_uint64, []),
+    "amem_pool_reserve": (C.c_int, [C.c_uint64]),
     "amem_shutdown": (C.c_int, []),
     "amem_ipc_start": (C.c_int, []),
     "amem_get_slot": (C.c_int, []),

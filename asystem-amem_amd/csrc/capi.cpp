@@ -570,8 +570,8 @@ void amem_get_counters(amem_counters* out) {
 void amem_get_cycle_stats(amem_cycle_stats* out) {
   if (!out) return;
   memset(out, 0, sizeof(*out));
-  Ctx* c = ctx_or_null();
-  if (c && c->engine) *out = c->engine->stats();
+  if (!gpu_present()) return;
+  if (Engine* en = engine_if_exists(current_device())) *out = en->stats();
 }
 
 // ---- controls ----
@@ -639,14 +639,24 @@ int64_t amem_get_option(const char* name) {
 }
 
 uint64_t amem_pool_trim(void) {
+  if (!gpu_present()) return 0;
+  Engine* en = engine_if_exists(current_device());
+  if (!en) return 0;
   Ctx* c = ctx_or_null();
-  if (!c) return 0;
+  if (!c) return en->trim_pool();
   std::lock_guard<std::mutex> ls(c->structure);  // not while a pause or resume is running
   {
     std::lock_guard<std::mutex> lf(c->fields);
     if (c->paused) return 0;  // the pool holds the parked bytes
   }
-  return c->engine ? c->engine->trim_pool() : 0;
+  return en->trim_pool();
+}
+
+int amem_pool_reserve(uint64_t bytes) {
+  if (int e = need_gpu("amem_pool_reserve")) return e;
+  Engine* en = engine_for(current_device());
+  if (!en) return (int)hipErrorNoDevice;
+  return (int)en->reserve_pool(bytes);
 }
 
 int amem_shutdown(void) {

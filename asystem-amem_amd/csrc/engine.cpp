@@ -110,6 +110,17 @@ hipEvent_t Engine::event_at(size_t i) {
   return events_[i];
 }
 
+hipError_t Engine::reserve_pool(uint64_t bytes) {
+  std::lock_guard<std::mutex> busy(busy_);
+  hipError_t e = init();
+  if (e != hipSuccess) return e;
+  const uint64_t limit = (uint64_t)options().pool_limit_bytes;
+  if (limit && bytes > limit) return hipErrorOutOfMemory;
+  e = pool_->ensure(bytes);
+  stats_.slab_bytes = pool_->capacity();
+  return e;
+}
+
 uint64_t Engine::trim_pool() {
   std::lock_guard<std::mutex> busy(busy_);
   if (!pool_) return 0;
@@ -1262,6 +1273,12 @@ Engine* engine_for(int dev) {
   if (en->init() != hipSuccess) { delete en; return nullptr; }
   g_engines[dev] = en;
   return en;
+}
+
+Engine* engine_if_exists(int dev) {
+  if (dev < 0 || dev >= AMEM_MAX_DEVS) return nullptr;
+  std::lock_guard<std::mutex> lk(g_engines_mtx);
+  return g_engines[dev];
 }
 
 void destroy_engines() {

@@ -83,6 +83,7 @@ class Engine {
 
   amem_cycle_stats stats() const { return stats_; }
   uint64_t trim_pool();
+  hipError_t reserve_pool(uint64_t bytes);
 
   // Standalone kernel entry points (synchronous).
   hipError_t zero_scan(const amem_extent* ext, uint64_t n, uint8_t* flags, amem_chunk_sum* sums,
@@ -139,6 +140,8 @@ class Engine {
 // Engine of a device, created on first use. Returns nullptr (after an ERROR log) when no
 // GPU is present: there is no host fallback for the data path.
 Engine* engine_for(int dev);
+// The engine of a device if one has been created, else nullptr.
+Engine* engine_if_exists(int dev);
 void destroy_engines();
 
 }  // namespace amem

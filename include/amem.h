@@ -297,6 +297,10 @@ int64_t amem_get_option(const char* name);
 
 /* Release the pinned host pool (only while not paused). Returns bytes freed. */
 uint64_t amem_pool_trim(void);
+/* Grow the pinned host pool of the current device to at least `bytes` ahead of time, so that the
+ * first pause does not pay for pinning host memory (the reference creates its host buffers inside
+ * the first pause, amem_nccl.cpp:505-508). 0 ok, else a HIP error. No reference counterpart. */
+int amem_pool_reserve(uint64_t bytes);
 
 /* Tear the per-process context down to the state before the first tracked allocation:
  * registry emptied (nothing is unmapped or freed), pool released, IPC service stopped,

@@ -441,3 +441,22 @@ def test_first_pause_on_a_full_device(eng):
         for p in hogs:
             assert hip.hipFree(p) == 0
     regs.free()
+
+
+def test_pool_reserved_ahead_of_the_first_pause(eng):
+    """The pinned pool can be sized before the first pause; the pause then finds its room ready, and
+    trimming gives the same bytes back."""
+    lib = eng
+    assert lib.amem_pool_reserve(300 * MiB) == 0
+    reserved = H.cycle_stats(lib)["slab_bytes"]
+    assert reserved >= 300 * MiB
+    fp = Footprint(1, 23, max_regions=8, threads=4)
+    regs = H.Regions(lib, fp)
+    assert fp.total_bytes < 300 * MiB
+    assert lib.amem_mem_pause(0, 0) == 0
+    assert H.cycle_stats(lib)["slab_bytes"] == reserved
+    assert lib.amem_pool_trim() == 0                       # not while the pool holds parked bytes
+    assert lib.amem_mem_resume(0, 0) == 0
+    assert regs.mismatched_bytes() == 0
+    regs.free()
+    assert lib.amem_pool_trim() == reserved
