@@ -92,6 +92,8 @@ def main():
     from asystem_amem_amd.footprint import Footprint
 
     H.enable_env()
+    import __graft_entry__
+    __graft_entry__.ensure_built()      # loads what is built; compiles only if a library is missing
     lib = B.load()
     if lib.amem_device_count() < 1:
         sys.exit("bench.py needs a GPU")
