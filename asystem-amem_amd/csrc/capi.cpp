@@ -89,15 +89,19 @@ static void fill_info(uint64_t va, const Region& r, amem_region_info* o) {
 int amem_release_peer_mapping(uint64_t va) {
   Ctx* c = ctx_or_null();
   if (!c || !gpu_present()) return 1;
-  const int dev = current_device();
   uint64_t handle = 0;
   size_t size = 0;
   {
     std::lock_guard<std::mutex> lk(c->fields);
-    auto it = c->allocTable[dev].find(va);
-    if (it == c->allocTable[dev].end()) return 1;
-    handle = it->second.handle;
-    size = it->second.allocSz;
+    bool found = false;
+    for (int dev = 0; dev < AMEM_MAX_DEVS && !found; ++dev) {  // the service thread's device need not be the region's
+      auto it = c->allocTable[dev].find(va);
+      if (it == c->allocTable[dev].end()) continue;
+      handle = it->second.handle;
+      size = it->second.allocSz;
+      found = true;
+    }
+    if (!found) return 1;
   }
   if (!handle) handle = vmm_handle_of(va);
   return (int)vmm_unmap_release(va, size, handle, 0);
@@ -296,23 +300,25 @@ int amem_add_peer_info(uint64_t src_va, uint64_t peer_va, int peer_dev) {
   return ret;
 }
 
+// The two handlers below run on the service thread, whose current device is the one the service
+// was started on; a process that drives several GPUs keeps one table per device, so the entry is
+// looked for in all of them (addresses and handles are unique within a process).
 int amem_register_peer_info(uint64_t src_handle, uint64_t peer_va, int peer_dev) {
   Ctx* c = ctx_or_null();
   int ret = 1;
   if (c && peer_dev >= 0 && peer_dev < AMEM_MAX_DEVS) {
-    const int dev = current_device();
     std::lock_guard<std::mutex> lf(c->fields);
-    auto ht = c->handleTable[dev].find(src_handle);
-    if (ht != c->handleTable[dev].end()) {
+    for (int dev = 0; dev < AMEM_MAX_DEVS && ret; ++dev) {
+      auto ht = c->handleTable[dev].find(src_handle);
+      if (ht == c->handleTable[dev].end()) continue;
       auto it = c->allocTable[dev].find(ht->second);
-      if (it != c->allocTable[dev].end()) {
-        it->second.peers[peer_dev] = peer_va;
-        it->second.hasPeer = true;
-        ret = 0;
-        LOGGER(DEBUG, "groupID:%d pid:%d localDptr:%llx localHandle:%llx register peer:%d peerPtr:%llx done",
-               amem_groupID, getpid(), (unsigned long long)ht->second, (unsigned long long)src_handle, peer_dev,
-               (unsigned long long)peer_va);
-      }
+      if (it == c->allocTable[dev].end()) continue;
+      it->second.peers[peer_dev] = peer_va;
+      it->second.hasPeer = true;
+      ret = 0;
+      LOGGER(DEBUG, "groupID:%d pid:%d localDptr:%llx localHandle:%llx register peer:%d peerPtr:%llx done",
+             amem_groupID, getpid(), (unsigned long long)ht->second, (unsigned long long)src_handle, peer_dev,
+             (unsigned long long)peer_va);
     }
   }
   if (ret)
@@ -324,18 +330,22 @@ int amem_register_peer_info(uint64_t src_handle, uint64_t peer_va, int peer_dev)
 int amem_update_peer_info(uint64_t va, int shared_fd) {
   Ctx* c = ctx_or_null();
   if (!c) { if (shared_fd >= 0) close(shared_fd); return 1; }
-  const int dev = current_device();
+  int dev = -1;
   size_t size = 0;
   {
     std::lock_guard<std::mutex> lf(c->fields);
-    auto it = c->allocTable[dev].find(va);
-    if (it == c->allocTable[dev].end()) {
-      LOGGER(ERROR, "groupID:%d pid:%d failed to find info for dptr:%llx to remap fd:%x", amem_groupID, getpid(),
-             (unsigned long long)va, shared_fd);
-      if (shared_fd >= 0) close(shared_fd);
-      return 1;
+    for (int d = 0; d < AMEM_MAX_DEVS && dev < 0; ++d) {
+      auto it = c->allocTable[d].find(va);
+      if (it == c->allocTable[d].end()) continue;
+      dev = d;
+      size = it->second.allocSz;
     }
-    size = it->second.allocSz;
+  }
+  if (dev < 0) {
+    LOGGER(ERROR, "groupID:%d pid:%d failed to find info for dptr:%llx to remap fd:%x", amem_groupID, getpid(),
+           (unsigned long long)va, shared_fd);
+    if (shared_fd >= 0) close(shared_fd);
+    return 1;
   }
   if (!gpu_present()) {
     LOGGER(ERROR, "pid:%d no HIP device: cannot import fd:%d", getpid(), shared_fd);
