@@ -6,6 +6,7 @@ import os
 import re
 import subprocess
 
+import numpy as np
 import pytest
 
 import oracle as O
@@ -258,3 +259,69 @@ def test_rccl_hook_library_exports_the_interposed_calls():
                      "amem_rccl_hook_registered"}
     # unversioned definitions: they satisfy librccl's versioned references (hipMemMap@hip_5.1 ...)
     assert "@" not in "".join(names)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_random_registry_sequences_match_oracle(fresh, fresh_orc, seed):
+    """Seeded random sequences of every registry call, the same call to the engine and to the oracle:
+    same return code each time, and the same table and counters after every batch. Addresses and handles
+    are made up (no GPU is touched); imported mappings use the two owner values both sides can judge
+    without a second process (own slot: refused; unknown owner: dropped)."""
+    lib, orc = fresh, fresh_orc
+    p = both(lib, orc)
+    rng = np.random.default_rng(1000 + seed)
+    base = 0x7e0000000000
+    live, next_handle = [], [0x100]
+
+    def new_handle():
+        next_handle[0] += 7
+        return next_handle[0]
+
+    lib.amem_add_alloc_info(base - (1 << 30), 2 * MiB, 0, 0, 0x77, -1, 0, None, 0)      # the slot exists from here on
+    orc.oracle_add_alloc_info(0, base - (1 << 30), 2 * MiB, 0, 0, 0x77, -1, 0, 0, 0)
+    slot = lib.amem_get_slot()
+    for step in range(600):
+        op = rng.integers(0, 100)
+        if op < 40 or not live:                                    # add, sometimes over an existing address
+            again = live and rng.integers(0, 5) == 0
+            va = int(rng.choice(live)) if again else base + int(rng.integers(0, 1 << 20)) * (2 * MiB)
+            type_ = int(rng.choice([0, 0, 0, 1, 2, 3, 4]))
+            peer = {}
+            if type_ > 2:
+                peer = dict(peer_dev=int(rng.choice([slot if slot >= 0 else 0, -1])), peer_handle=0x55)
+            rc = p.add(va, int(rng.integers(1, 64)) * 64 * 1024, type_=type_, handle=new_handle(),
+                       caller=int(rng.choice([0, 1, 2, 3, 7, 10, 15, 16, 40])), user=int(rng.integers(0, 2)) * 0xABC, **peer)
+            if rc == 0 and va not in live:
+                live.append(va)
+            elif rc != 0 and va in live:
+                live.remove(va)          # a failed import over a known address erases the entry (amem_nccl.cpp:214-219)
+        elif op < 60:                                              # delete: known or unknown, handle given or not
+            va = int(rng.choice(live)) if rng.integers(0, 4) else base + 12345 * 4096
+            h = 0
+            if rng.integers(0, 2):
+                t = H.region_table(lib, 0).get(va)
+                h = t["handle"] if t else 0x999
+            a = lib.amem_del_alloc_info(va, h, int(rng.choice([-1, 0, 3])))
+            b = orc.oracle_del_alloc_info(0, va, h, 0)
+            assert a == b
+            if va in live:
+                live.remove(va)
+        elif op < 72:
+            va = int(rng.choice(live)) if rng.integers(0, 4) else 0x4242
+            n = int(rng.integers(1, 4))
+            assert lib.amem_add_refcount(C.c_void_p(va), n) == orc.oracle_add_refcount(0, va, n)
+        elif op < 84:
+            va = int(rng.choice(live)) if rng.integers(0, 4) else 0x4242
+            dev, pva = int(rng.integers(0, 8)), 0x5000 + int(rng.integers(0, 99)) * 4096
+            assert lib.amem_add_peer_info(va, pva, dev) == orc.oracle_add_peer_info(0, va, pva, dev)
+        elif op < 96:
+            t = H.region_table(lib, 0)
+            h = t[int(rng.choice(live))]["handle"] if rng.integers(0, 4) else 0xBAD
+            dev, pva = int(rng.integers(0, 8)), 0x9000 + int(rng.integers(0, 99)) * 4096
+            assert lib.amem_register_peer_info(h, pva, dev) == orc.oracle_register_peer_info(0, h, pva, dev)
+        else:
+            g = int(rng.integers(0, 1000))
+            assert lib.amem_set_group_id(g) == orc.oracle_set_group_id(0, g) == 1      # too late: a context exists
+        if step % 50 == 49:
+            p.check()
+    p.check()

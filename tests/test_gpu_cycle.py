@@ -460,3 +460,97 @@ def test_pool_reserved_ahead_of_the_first_pause(eng):
     assert regs.mismatched_bytes() == 0
     regs.free()
     assert lib.amem_pool_trim() == reserved
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_random_sequences_with_cycles_match_oracle(eng, fresh_orc, seed):
+    """A seeded random life of a process — allocations of ragged sizes coming and going, writes,
+    pause/resume cycles at arbitrary points, registrations refused and regions dropped while paused —
+    played to the engine on the GPU and to the oracle in host memory. After every cycle the bytes of
+    every live region equal the mirror kept here, on both sides, and the two registries agree."""
+    lib, orc = eng, fresh_orc
+    rng = np.random.default_rng(77 + seed)
+    live = []          # dicts: eva, ealloc, ova, size, data (the mirror)
+
+    def new_region():
+        size = int(rng.integers(1, 96)) * CHUNK + int(rng.choice([0, 0, 16, 4096, 65520]))
+        data = rng.integers(0, 256, size, dtype=np.uint8)
+        for c in range(0, size, CHUNK):                                     # about a third of the chunks zero
+            if rng.integers(0, 3) == 0:
+                data[c:c + CHUNK] = 0
+        caller = int(rng.choice([B.CALLER_P2P, 0, 3]))
+        va, h, asz = C.c_uint64(), C.c_uint64(), C.c_uint64()
+        assert lib.amem_vmm_alloc(size, 0, C.byref(va), C.byref(h), C.byref(asz)) == 0
+        pad = np.zeros(asz.value, dtype=np.uint8)
+        pad[:size] = data
+        assert lib.amem_copy_to_device(va.value, pad.ctypes.data, pad.nbytes) == 0
+        ova, oh, oasz = C.c_uint64(), C.c_uint64(), C.c_uint64()
+        assert orc.oracle_vmm_alloc(size, C.byref(ova), C.byref(oh), C.byref(oasz)) == 0
+        assert oasz.value == asz.value
+        np.frombuffer((C.c_uint8 * asz.value).from_address(ova.value), dtype=np.uint8)[:] = pad
+        a = lib.amem_add_alloc_info(va.value, asz.value, B.TYPE_LOCAL, 0, h.value, -1, 0, None, caller)
+        b = orc.oracle_add_alloc_info(0, ova.value, oasz.value, B.TYPE_LOCAL, 0, oh.value, -1, 0, 0, caller)
+        assert a == b
+        r = dict(eva=va.value, ealloc=asz.value, ova=ova.value, data=pad, tracked=(a == 0))
+        if a == 0:
+            live.append(r)
+        else:                                                              # refused (paused): nobody tracks it
+            assert lib.amem_vmm_free(va.value, asz.value, h.value) == 0
+            assert orc.oracle_vmm_free(ova.value, oasz.value, oh.value) == 0
+        return a
+
+    def drop(r, paused):
+        assert lib.amem_del_alloc_info(r["eva"], 0, 0) == orc.oracle_del_alloc_info(0, r["ova"], 0, 0) == 0
+        assert lib.amem_vmm_free(r["eva"], r["ealloc"], 0) == 0
+        assert orc.oracle_vmm_free(r["ova"], r["ealloc"], 0) == 0
+        live.remove(r)
+
+    def check_all():
+        same_as_oracle(lib, orc, [r["eva"] for r in live], [(r["ova"], r["ealloc"]) for r in live])
+        for r in live:
+            got = np.empty(r["ealloc"], dtype=np.uint8)
+            assert lib.amem_copy_from_device(got.ctypes.data, r["eva"], got.nbytes) == 0
+            assert np.array_equal(got, r["data"])
+            ogot = np.frombuffer((C.c_uint8 * r["ealloc"]).from_address(r["ova"]), dtype=np.uint8)
+            assert np.array_equal(ogot, r["data"])
+
+    for _ in range(6):
+        assert new_region() == 0
+    cycles = 0
+    for step in range(70):
+        op = rng.integers(0, 100)
+        if op < 30 and len(live) < 40:
+            assert new_region() == 0
+        elif op < 45 and len(live) > 2:
+            drop(live[int(rng.integers(0, len(live)))], False)
+        elif op < 70 and live:
+            r = live[int(rng.integers(0, len(live)))]
+            a = int(rng.integers(0, r["ealloc"] // 16)) * 16
+            n = min(int(rng.integers(1, 40000)) * 16, r["ealloc"] - a)
+            patch = rng.integers(0, 256, n, dtype=np.uint8) if rng.integers(0, 3) else np.zeros(n, dtype=np.uint8)
+            r["data"][a:a + n] = patch
+            assert lib.amem_copy_to_device(r["eva"] + a, patch.ctypes.data, n) == 0
+            np.frombuffer((C.c_uint8 * n).from_address(r["ova"] + a), dtype=np.uint8)[:] = patch
+        else:
+            assert lib.amem_mem_pause(0, 0) == orc.oracle_mem_pause(0) == 0
+            same_as_oracle(lib, orc, [r["eva"] for r in live], [(r["ova"], r["ealloc"]) for r in live])
+            if rng.integers(0, 3) == 0:
+                assert new_region() == 1                                   # refused on both sides while paused
+            gone = None
+            if rng.integers(0, 3) == 0 and len(live) > 2:
+                gone = live[int(rng.integers(0, len(live)))]               # forgotten while paused: it stays a hole
+                assert lib.amem_del_alloc_info(gone["eva"], 0, 0) == orc.oracle_del_alloc_info(0, gone["ova"], 0, 0) == 0
+                live.remove(gone)
+            assert lib.amem_mem_resume(0, 0) == orc.oracle_mem_resume(0) == 0
+            if gone:                                                       # nothing is mapped there: only the address goes
+                assert lib.amem_vmm_free(gone["eva"], gone["ealloc"], 0) == 0
+                assert orc.oracle_vmm_free(gone["ova"], gone["ealloc"], 0) == 0
+            cycles += 1
+            check_all()
+    assert cycles >= 5
+    assert lib.amem_mem_pause(0, 0) == orc.oracle_mem_pause(0) == 0
+    assert lib.amem_mem_resume(0, 0) == orc.oracle_mem_resume(0) == 0
+    check_all()
+    for r in list(live):
+        drop(r, False)
+    assert lib.amem_region_count(0) == 0
