@@ -373,15 +373,19 @@ hipError_t Engine::release_local(Ctx& c, Region* r, uint64_t va, std::pair<uint6
   if (r->type == AMEM_TYPE_LOCAL_SYMM)
     LOGGER(DEBUG, "memPause: dptr:%llx is symmetric memory; no multicast object to unbind on this platform",
            (unsigned long long)va);
+  // The reference drops `refcount` extra references here, one per retain its callers reported
+  // (amem_nccl.cpp:541-549). On this runtime a retain takes no reference, so there are none to
+  // drop, and a release beyond the creator's would touch a handle that is already freed. The
+  // count is kept in the record and reported; no extra release is issued.
   if (r->refcount > 0)
-    LOGGER(DEBUG, "memPause: groupID:%d pid:%d dptr:%llx refcount:%d", amem_groupID_value(), getpid(),
-           (unsigned long long)va, r->refcount);
+    LOGGER(DEBUG, "memPause: groupID:%d pid:%d dptr:%llx refcount:%d (no extra releases on this runtime)",
+           amem_groupID_value(), getpid(), (unsigned long long)va, r->refcount);
   hipError_t e;
   if (deferred) {
     e = vmm_unmap(va, r->allocSz);
-    *deferred = {old, r->refcount};
+    *deferred = {old, 0};
   } else {
-    e = vmm_unmap_release(va, r->allocSz, old, r->refcount);
+    e = vmm_unmap_release(va, r->allocSz, old, 0);
   }
   {
     std::lock_guard<std::mutex> lk(c.fields);

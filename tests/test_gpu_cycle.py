@@ -554,3 +554,28 @@ def test_random_sequences_with_cycles_match_oracle(eng, fresh_orc, seed):
     for r in list(live):
         drop(r, False)
     assert lib.amem_region_count(0) == 0
+
+
+def test_reported_retains_do_not_cause_extra_releases(eng):
+    """amem_add_refcount records retains the caller says it holds. The reference releases that many extra
+    times at pause (amem_nccl.cpp:542-546); on this runtime a retain takes no reference, so the engine
+    must not, and the memory must still be freed by the pause and come back intact."""
+    lib = eng
+    fp = Footprint(1, 29, max_regions=4, threads=2)
+    regs = H.Regions(lib, fp)
+    h = C.c_void_p()
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMemRetainAllocationHandle.argtypes = [C.POINTER(C.c_void_p), C.c_void_p]
+    for i in range(2):                                                  # what a caller of the hook would have done
+        assert hip.hipMemRetainAllocationHandle(C.byref(h), C.c_void_p(int(regs.va[i]))) == 0
+        assert h.value == int(regs.handle[i])
+        assert lib.amem_add_refcount(C.c_void_p(int(regs.va[i])), 2) == 0
+    assert lib.amem_mem_pause(0, 0) == 0 and lib.amem_mem_resume(0, 0) == 0      # warm
+    for _ in range(2):
+        free0 = H.mem_free(lib)
+        assert lib.amem_mem_pause(0, 0) == 0
+        assert H.mem_free(lib) - free0 >= fp.total_bytes - 4 * MiB
+        assert lib.amem_mem_resume(0, 0) == 0
+        assert regs.mismatched_bytes() == 0
+    assert regs.table()[int(regs.va[0])]["refcount"] == 2               # the record keeps what it was told
+    regs.free()
