@@ -265,6 +265,7 @@ int amem_set_enabled(int on);
  *                     3 = many short pack launches into pinned host memory, confined to
  *                         "pause_xcds" XCDs and "pause_wgs" workgroups, while a second host
  *                         thread unmaps each group of regions as soon as its launch is done
+ *                         (and a third releases their handles, see "release_thread")
  *                     2 = the default, currently 3
  *                     4 = measurement aid: the reference's own structure in HIP calls (one waited-for
  *                         whole-region hipMemcpyAsync per region each way, no scan, no elision)
@@ -275,7 +276,10 @@ int amem_set_enabled(int on);
  *   "dma_min_bytes"   extents at least this long use hipMemcpyAsync in the direct path
  *   "staging_bytes"   size of each of the two device staging buffers
  *   "slab_bytes"      size of one pinned host slab (power of two)
- *   "link_wgs"        workgroups of a kernel that reads or writes host memory
+ *   "link_wgs"        workgroups of a kernel that reads or writes host memory (default 96)
+ *   "hbm_wgs"         most workgroups of a kernel that touches device memory only (default 65536)
+ *   "resume_batch_bytes" resume maps regions in batches of about this many bytes and follows each
+ *                     batch with one unpack launch (default 64 MiB)
  *   "peer_timeout_ms" how long resume waits for owners before failing (0 = forever)
  *   "offload_free_tag" caller tag (0-15, -1 = none) whose regions hold scratch data: pause releases
  *                     them without copying and resume hands them back zero-filled. This is what
