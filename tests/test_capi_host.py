@@ -277,6 +277,7 @@ def test_random_registry_sequences_match_oracle(fresh, fresh_orc, seed):
         next_handle[0] += 7
         return next_handle[0]
 
+    assert lib.amem_set_group_id(300 + seed) == orc.oracle_set_group_id(0, 300 + seed) == 0   # before the first allocation
     lib.amem_add_alloc_info(base - (1 << 30), 2 * MiB, 0, 0, 0x77, -1, 0, None, 0)      # the slot exists from here on
     orc.oracle_add_alloc_info(0, base - (1 << 30), 2 * MiB, 0, 0, 0x77, -1, 0, 0, 0)
     slot = lib.amem_get_slot()
