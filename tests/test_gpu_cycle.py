@@ -2,6 +2,7 @@
 table and counters equal to the oracle's after the same calls, physical memory really released,
 every option path, and the edge cases of the reference's state machine."""
 import ctypes as C
+import os
 
 import numpy as np
 import pytest
@@ -579,3 +580,23 @@ def test_reported_retains_do_not_cause_extra_releases(eng):
         assert regs.mismatched_bytes() == 0
     assert regs.table()[int(regs.va[0])]["refcount"] == 2               # the record keeps what it was told
     regs.free()
+
+
+def test_native_caller_through_the_reference_api(gpu, tmp_path):
+    """A C++ program that knows only include/amem_nccl.h (the reference's names and default arguments)
+    and the HIP virtual-memory API allocates, registers, pauses, resumes, checks its bytes through the
+    pointers it kept, and frees by address: the drop-in boundary exercised natively on the GPU."""
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    libdir = os.path.dirname(B.LIB_PATH)
+    exe = str(tmp_path / "cxx_cycle_on_gpu")
+    subprocess.run(["g++", "-O1", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-D__HIP_PLATFORM_AMD__",
+                    "-I", os.path.join(root, "include"), "-I", os.path.join(rocm, "include"),
+                    os.path.join(root, "tests", "link_check", "cxx_cycle_on_gpu.cpp"), "-o", exe, B.LIB_PATH,
+                    "-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath," + libdir],
+                   check=True, capture_output=True, text=True)
+    env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="3", AMEM_IPC="0")
+    r = subprocess.run([exe], env=env, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and "c++ cycle on the gpu ok" in r.stdout, (r.returncode, r.stdout[-3000:], r.stderr[-3000:])
+    assert "memPause: pause results." in r.stdout and "offload:4" in r.stdout      # the reference's summary line
