@@ -600,3 +600,53 @@ def test_native_caller_through_the_reference_api(gpu, tmp_path):
     r = subprocess.run([exe], env=env, capture_output=True, text=True, timeout=120)
     assert r.returncode == 0 and "c++ cycle on the gpu ok" in r.stdout, (r.returncode, r.stdout[-3000:], r.stderr[-3000:])
     assert "memPause: pause results." in r.stdout and "offload:4" in r.stdout      # the reference's summary line
+
+
+def test_hook_and_inspection_calls_from_another_thread_during_cycles(eng):
+    """The allocator hook and the inspection calls come from arbitrary threads (NCCL's proxy thread among
+    them) while the main thread pauses and resumes. A second thread keeps calling them for the length of
+    eight cycles; nothing deadlocks, every answer is one of the legal ones, and the bytes survive."""
+    import threading
+    lib = eng
+    fp = Footprint(2, 31, max_regions=48, threads=8)
+    regs = H.Regions(lib, fp)
+    vas = [int(v) for v in regs.va]
+    stop, seen, errors = threading.Event(), {"paused": 0, "calls": 0}, []
+
+    def other_thread():
+        info = B.RegionInfo()
+        k = 0
+        try:
+            while not stop.is_set():
+                p = lib.amem_check_paused(0)
+                seen["paused"] += p
+                n = lib.amem_region_count(0)
+                assert n == len(vas), n
+                if lib.amem_region_find(0, vas[k % len(vas)], C.byref(info)) == 0:
+                    assert info.state in (B.STATE_ALLOC, B.STATE_OFFLOADING, B.STATE_HOLE, B.STATE_PRELOADING)
+                    assert info.alloc_sz == int(regs.alloc[k % len(vas)])
+                H.counters(lib)
+                # two hook-side writers of region fields (they take the same lock as the engine's updates)
+                rc = lib.amem_add_refcount(C.c_void_p(vas[k % len(vas)]), 0)
+                assert rc == 0
+                assert lib.amem_add_peer_info(vas[k % len(vas)], 0, 5) == 0        # peer address 0 = no peer
+                seen["calls"] += 1
+                k += 1
+        except Exception as e:                                                   # surfaced by the main thread
+            errors.append(repr(e))
+
+    t = threading.Thread(target=other_thread)
+    t.start()
+    try:
+        for cyc in range(8):
+            touched = fp.mutate(cyc)
+            regs.write_chunks(touched)
+            assert lib.amem_mem_pause(0, 0) == 0
+            assert lib.amem_mem_resume(0, 0) == 0
+    finally:
+        stop.set()
+        t.join(60)
+    assert not t.is_alive() and errors == []
+    assert seen["calls"] > 100 and seen["paused"] > 0
+    assert regs.mismatched_bytes() == 0
+    regs.free()
