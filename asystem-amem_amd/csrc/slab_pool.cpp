@@ -16,8 +16,11 @@ SlabPool::~SlabPool() { trim(); }
 hipError_t SlabPool::ensure(uint64_t bytes) {
   while (capacity() < bytes) {
     void* p = nullptr;
-    // Default flags: coherent / non-coherent / portable / NUMA-user variants measured the same
-    // for both the copy engine and kernels that read or write the slab.
+    // Default flags. Without hipHostMallocNumaUser the runtime places pinned memory on the NUMA
+    // node closest to the current device, which is the placement the reference asks for by hand
+    // (amem_allocHost, amem_nccl.h:251-267: the GPU's node, else node 0); the caller's current
+    // device is the engine's device here. Coherent / non-coherent / portable variants measured
+    // the same for both the copy engine and kernels that read or write the slab.
     hipError_t e = CHECK_HIP(hipHostMalloc(&p, slab_bytes_, hipHostMallocDefault));
     if (e != hipSuccess) return e;
     slabs_.push_back((uint8_t*)p);
