@@ -762,6 +762,27 @@ int Engine::pause(Ctx& c, bool* rolled_back) {
         invalid.push_back(&r);
         continue;
       }
+      // The handle is read off the mapping, as the reference does at this point
+      // (amem_nccl.cpp:539-540): the one given at registration is only as good as the caller's
+      // bookkeeping, and releasing a stale one would touch freed memory.
+      const uint64_t mapped = vmm_handle_of(kv.first);
+      if (mapped == 0) {
+        LOGGER(ERROR, "memPause: groupID:%d pid:%d dptr:%llx allocSz:%ld is not memory of the virtual-memory API; "
+               "it cannot be released and is left alone", amem_groupID_value(), getpid(),
+               (unsigned long long)kv.first, (long)r.allocSz);
+        if (rc == 0) rc = (int)hipErrorInvalidValue;
+        invalid.push_back(&r);
+        continue;
+      }
+      if (mapped != r.handle) {
+        LOGGER(WARN, "memPause: groupID:%d pid:%d dptr:%llx was registered with handle %llx but is mapped to %llx; "
+               "using the mapping's", amem_groupID_value(), getpid(), (unsigned long long)kv.first,
+               (unsigned long long)r.handle, (unsigned long long)mapped);
+        std::lock_guard<std::mutex> lk(c.fields);
+        c.handleTable[dev_].erase(r.handle);
+        r.handle = mapped;
+        c.handleTable[dev_].emplace(mapped, kv.first);
+      }
       locals.push_back(&r);
       segs_.push_back({kv.first, (uint64_t)r.allocSz});
     }
@@ -904,7 +925,9 @@ int Engine::pause(Ctx& c, bool* rolled_back) {
   if (rc == 0) {
     for (auto& kv : table) {
       Region& r = kv.second;
-      if (!from_peer(r.type) && r.state != AMEM_STATE_HOLE) note(release_local(c, &r, kv.first));
+      if (from_peer(r.type) || r.state == AMEM_STATE_HOLE) continue;
+      if (std::find(invalid.begin(), invalid.end(), &r) != invalid.end()) continue;  // reported above, left as found
+      note(release_local(c, &r, kv.first));
     }
   } else {
     LOGGER(ERROR, "memPause: groupID:%d pid:%d GPU:%d failed with HIP error %d; physical memory of "

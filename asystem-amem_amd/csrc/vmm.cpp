@@ -66,7 +66,27 @@ hipError_t vmm_alloc(size_t bytes, int dev, uint64_t* va, uint64_t* handle, size
 // handle without taking a reference (measured: memory is freed by the first release after
 // an unmap even when a retain came before), so the matching release must NOT be issued: it
 // would drop the creator's reference.
+// hipMemRetainAllocationHandle must only see addresses mapped through the virtual-memory API:
+// given ordinary hipMalloc memory it crashes inside the runtime (measured on ROCm 7.2), while
+// hipMemGetAccess answers with an error for such memory and for reserved-but-unmapped
+// addresses alike. So the access query goes first.
+bool vmm_is_mapped(uint64_t va) {
+  if (va == 0) return false;
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  hipMemLocation loc;
+  loc.type = hipMemLocationTypeDevice;
+  loc.id = dev;
+  unsigned long long flags = 0;
+  if (hipMemGetAccess(&flags, &loc, (void*)(uintptr_t)va) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return true;
+}
+
 uint64_t vmm_handle_of(uint64_t va) {
+  if (!vmm_is_mapped(va)) return 0;
   hipMemGenericAllocationHandle_t h = nullptr;
   if (hipMemRetainAllocationHandle(&h, (void*)(uintptr_t)va) != hipSuccess || !h) {
     (void)hipGetLastError();

@@ -46,7 +46,9 @@ hipError_t vmm_import_map(int dev, uint64_t va, size_t size, int fd, bool close_
                           uint64_t* new_handle);
 // Allocation or mapping that contains `addr`: its base and size. False when the runtime knows none.
 bool vmm_range_of(uint64_t addr, uint64_t* base, uint64_t* size);
-// Handle currently mapped at `va`, 0 if none. Takes no reference.
+// True when `va` is mapped through the virtual-memory API (safe to ask about any address).
+bool vmm_is_mapped(uint64_t va);
+// Handle currently mapped at `va`; 0 if none or if `va` is not virtual-memory-API memory. Takes no reference.
 uint64_t vmm_handle_of(uint64_t va);
 // Device that owns the physical memory behind `handle`, -1 if unknown.
 int vmm_handle_device(uint64_t handle);

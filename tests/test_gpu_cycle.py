@@ -318,7 +318,7 @@ def test_stale_registration_is_reported_not_read(eng):
     assert np.array_equal(out, data)
     lib.amem_del_alloc_info(good[0].value, 0, 0)
     lib.amem_vmm_free(good[0].value, good[2].value, 0)
-    lib.amem_vmm_free(bad[0].value, bad[2].value, 0)                   # pause unmapped it; the reservation is freed here
+    lib.amem_vmm_free(bad[0].value, bad[2].value, 0)                   # the pause left it alone: still mapped
     # the kernels' own entry points refuse ranges the runtime does not know
     ext = (B.Extent * 1)(B.Extent(0x7e0000000000, 65536))
     one = (C.c_uint8 * 1)()
@@ -648,5 +648,49 @@ def test_hook_and_inspection_calls_from_another_thread_during_cycles(eng):
         t.join(60)
     assert not t.is_alive() and errors == []
     assert seen["calls"] > 100 and seen["paused"] > 0
+    assert regs.mismatched_bytes() == 0
+    regs.free()
+
+
+def test_wrong_handles_and_foreign_memory_at_registration(eng):
+    """What the caller says at registration is not trusted where a mistake would free the wrong thing:
+    a region registered with a handle value that is not the mapping's is paused with the mapping's own
+    handle, and memory that does not come from the virtual-memory API (nothing can unmap it) is
+    reported and left exactly as it is while the other regions cycle."""
+    lib = eng
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+    hip.hipFree.argtypes = [C.c_void_p]
+    fp = Footprint(2, 37, max_regions=3, threads=2)
+    regs = H.Regions(lib, fp, register=False)
+    rng = np.random.default_rng(9)
+    # region 0: right handle; region 1: a made-up handle value; region 2: no handle given at all
+    assert lib.amem_add_alloc_info(int(regs.va[0]), int(regs.alloc[0]), 0, 0, int(regs.handle[0]), -1, 0, None, 1) == 0
+    assert lib.amem_add_alloc_info(int(regs.va[1]), int(regs.alloc[1]), 0, 0, 0x1234560, -1, 0, None, 1) == 0
+    assert lib.amem_add_alloc_info(int(regs.va[2]), int(regs.alloc[2]), 0, 0, 0, -1, 0, None, 1) == 0
+    regs.registered = True
+    plain = C.c_void_p()
+    assert hip.hipMalloc(C.byref(plain), 4 * MiB) == 0
+    mine = rng.integers(1, 256, 4 * MiB, dtype=np.uint8)
+    assert lib.amem_copy_to_device(plain.value, mine.ctypes.data, mine.nbytes) == 0
+    assert lib.amem_add_alloc_info(plain.value, 4 * MiB, 0, 0, 0xBEEF0, -1, 0, None, 1) == 0
+    free0 = H.mem_free(lib)
+    assert lib.amem_mem_pause(0, 0) != 0                                  # reported ...
+    assert lib.amem_check_paused(0) == 1                                  # ... and the rest is paused
+    st = H.cycle_stats(lib)
+    assert st["local_regions"] == 3
+    tab = H.region_table(lib, 0)
+    assert tab[plain.value]["state"] == B.STATE_ALLOC
+    assert all(tab[int(v)]["state"] == B.STATE_HOLE for v in regs.va)
+    got = np.empty(4 * MiB, dtype=np.uint8)
+    assert lib.amem_copy_from_device(got.ctypes.data, plain.value, got.nbytes) == 0 and np.array_equal(got, mine)
+    assert lib.amem_mem_resume(0, 0) == 0 and lib.amem_check_paused(0) == 0
+    assert regs.mismatched_bytes() == 0
+    assert lib.amem_copy_from_device(got.ctypes.data, plain.value, got.nbytes) == 0 and np.array_equal(got, mine)
+    tab = H.region_table(lib, 0)
+    assert all(tab[int(v)]["handle"] not in (0, 0x1234560) for v in regs.va)
+    assert lib.amem_del_alloc_info(plain.value, 0xBEEF0, 0) == 0
+    assert hip.hipFree(plain) == 0
+    assert lib.amem_mem_pause(0, 0) == 0 and lib.amem_mem_resume(0, 0) == 0     # with the foreign entry gone: clean
     assert regs.mismatched_bytes() == 0
     regs.free()
