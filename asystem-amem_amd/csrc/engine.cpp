@@ -787,8 +787,8 @@ int Engine::pause(Ctx& c, bool* rolled_back) {
       segs_.push_back({kv.first, (uint64_t)r.allocSz});
     }
   }
-  const int rc_validation = rc;
-  rc = 0;  // the valid regions are still paused; the validation error is returned at the end
+  int rc_soft = rc;  // errors that concern single regions: the others are still paused, the error is returned at the end
+  rc = 0;
 
   stats_.peer_regions = imported.size();
   stats_.local_regions = locals.size();
@@ -885,10 +885,17 @@ int Engine::pause(Ctx& c, bool* rolled_back) {
     auto tu = Clock::now();
     Region* r = pr.second;
     LOGGER(DEBUG, "memPause: release peer handle %llx.", (unsigned long long)pr.first);
-    uint64_t h = r->handle ? r->handle : vmm_handle_of(pr.first);
+    const uint64_t h = vmm_handle_of(pr.first);  // the mapping's own, as for local regions
+    if (h == 0) {
+      LOGGER(ERROR, "memPause: groupID:%d pid:%d imported dptr:%llx is not mapped; left alone", amem_groupID_value(),
+             getpid(), (unsigned long long)pr.first);
+      if (rc_soft == 0) rc_soft = (int)hipErrorInvalidValue;
+      continue;
+    }
     note(vmm_unmap_release(pr.first, r->allocSz, h, 0));
     std::lock_guard<std::mutex> lk(c.fields);
     r->state = AMEM_STATE_HOLE;
+    r->handle = 0;
     c.releaseShadowCnt++;
     stats_.pause_unmap_ms += ms_since(tu);
   }
@@ -942,7 +949,7 @@ int Engine::pause(Ctx& c, bool* rolled_back) {
          amem_groupID_value(), getpid(), dev_, (long)c.pauseCnt, (long)((total - free_sz) >> 20),
          (long)(stats_.footprint_bytes >> 20), (long)stats_.pause_ms, c.offloadCnt, c.releaseLocalCnt,
          c.releaseShadowCnt);
-  return rc ? rc : rc_validation;
+  return rc ? rc : rc_soft;
 }
 
 void Engine::forget(uint64_t va) {
