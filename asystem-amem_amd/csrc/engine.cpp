@@ -941,14 +941,19 @@ int Engine::pause(Ctx& c, bool* rolled_back) {
            "regions not yet released stays mapped", amem_groupID_value(), getpid(), dev_, rc);
   }
   note(CHECK_HIP(hipStreamSynchronize(dstream_)));
-  c.pauseCnt++;
+  long n_pause;
+  int n_offload, n_local, n_shadow;
+  {
+    std::lock_guard<std::mutex> lk(c.fields);
+    n_pause = (long)++c.pauseCnt;
+    n_offload = c.offloadCnt; n_local = c.releaseLocalCnt; n_shadow = c.releaseShadowCnt;
+  }
   stats_.pause_ms = ms_since(t0);
   (void)CHECK_HIP(hipMemGetInfo(&free_sz, &total));
   LOGGER(INFO, "memPause: pause results. groupID:%d pid:%d GPU:%d pauseCnt:%ld memUsed:%ld MB after paused, "
          "released:%ld MB, duration:%ld ms offload:%d releaseLocal:%d releasePeer:%d",
-         amem_groupID_value(), getpid(), dev_, (long)c.pauseCnt, (long)((total - free_sz) >> 20),
-         (long)(stats_.footprint_bytes >> 20), (long)stats_.pause_ms, c.offloadCnt, c.releaseLocalCnt,
-         c.releaseShadowCnt);
+         amem_groupID_value(), getpid(), dev_, n_pause, (long)((total - free_sz) >> 20),
+         (long)(stats_.footprint_bytes >> 20), (long)stats_.pause_ms, n_offload, n_local, n_shadow);
   return rc ? rc : rc_soft;
 }
 
@@ -1222,10 +1227,17 @@ int Engine::resume(Ctx& c, bool* incomplete) {
   }
   stats_.resume_ms = ms_since(t0);
   (void)CHECK_HIP(hipMemGetInfo(&free_sz, &total));
+  long n_resume;
+  int n_offload, n_local, n_shadow;
+  {
+    std::lock_guard<std::mutex> lk(c.fields);
+    n_resume = (long)(c.resumeCnt + 1);
+    n_offload = c.offloadCnt; n_local = c.releaseLocalCnt; n_shadow = c.releaseShadowCnt;
+  }
   LOGGER(INFO, "groupID:%d pid:%d GPU:%d resumeCnt:%ld memUsed:%ld MB after resumed, duration:%ld ms "
          "offloadLeft:%d releaseLocalLeft:%d releasePeerLeft:%d exportSz:%ld",
-         amem_groupID_value(), getpid(), dev_, (long)(c.resumeCnt + 1), (long)((total - free_sz) >> 20),
-         (long)stats_.resume_ms, c.offloadCnt, c.releaseLocalCnt, c.releaseShadowCnt, (long)(exportSz >> 20));
+         amem_groupID_value(), getpid(), dev_, n_resume, (long)((total - free_sz) >> 20),
+         (long)stats_.resume_ms, n_offload, n_local, n_shadow, (long)(exportSz >> 20));
   return rc;
 }
 
