@@ -218,8 +218,11 @@ def test_processes_sharing_one_gpu(gpu, world):
                     p.kill()
 
 
-def test_peer_path_in_loopback(gpu, fresh):
-    """The whole cross-process path inside one process: the process imports its own exported
+@pytest.mark.parametrize("nregions", [5, 256])
+def test_peer_path_in_loopback(gpu, fresh, nregions):
+    """(256 regions: the per-process layout of benchmark configuration 5, every region exported and
+    imported once, 256 descriptor messages per resume.)
+    The whole cross-process path inside one process: the process imports its own exported
     regions at second addresses and, with peer_loopback on, registers them with its own socket
     service as if it were another process. Pause must drop the imported mappings first and
     really free the memory; resume must re-create, re-export through the socket (SCM_RIGHTS)
@@ -229,8 +232,10 @@ def test_peer_path_in_loopback(gpu, fresh):
     lib = fresh
     assert lib.amem_set_option(b"peer_loopback", 1) == 0
     try:
-        fp = Footprint(2, 11, max_regions=5, threads=2)
+        fp = Footprint(2, 11 if nregions == 5 else 4, max_regions=nregions, threads=8)
         regs = H.Regions(lib, fp)
+        n = len(regs.va)
+        assert n == nregions
         slot = lib.amem_get_slot()
         assert slot >= 0
         imports = []
@@ -254,8 +259,8 @@ def test_peer_path_in_loopback(gpu, fresh):
 
         assert imports_match() == 0
         tab = H.region_table(lib, 0)
-        assert len(tab) == 10
-        for i in range(5):
+        assert len(tab) == 2 * n
+        for i in range(n):
             t = tab[int(regs.va[i])]
             assert t["has_peer"] == 1 and t["peers"][slot] == imports[i]
         c = H.counters(lib)
@@ -266,7 +271,7 @@ def test_peer_path_in_loopback(gpu, fresh):
         for cycle in range(2):
             assert lib.amem_mem_pause(0, 0) == 0
             c = H.counters(lib)
-            assert (c["offload_cnt"], c["release_local_cnt"], c["release_shadow_cnt"]) == (5, 5, 5)
+            assert (c["offload_cnt"], c["release_local_cnt"], c["release_shadow_cnt"]) == (n, n, n)
             assert H.mem_free(lib) - free0 >= fp.total_bytes - 8 * MiB      # both references are gone
             assert all(t["state"] == B.STATE_HOLE for t in H.region_table(lib, 0).values())
             assert lib.amem_mem_resume(0, 0) == 0
@@ -357,3 +362,4 @@ def test_owner_forgets_an_importer_whose_process_is_gone(gpu, fresh):
     assert lib.amem_mem_pause(0, 0) == 0 and H.counters(lib)["release_local_cnt"] == 0
     assert lib.amem_mem_resume(0, 0) == 0 and regs.mismatched_bytes() == 0
     regs.free()
+
