@@ -1,8 +1,8 @@
 """Several processes sharing the one GPU (benchmark configuration 5 at reduced size): every process
 owns regions, exports them as POSIX fds, imports all peers' regions; coordinated pause (importers
 let go first, owners' release then frees the memory) and resume (owners re-create and re-export,
-importers remap at their original VA). Reference: amem_nccl.cpp:517-526, :633-662, R10 of the
-hot-path table. Each process checks bytes at original VAs, counters, and that no fd leaks."""
+importers remap at their original VA). Reference: amem_nccl.cpp:517-526, :633-662;
+gmm_client_impl.cpp:479-532. Each process checks bytes at original VAs, counters, and that no fd leaks."""
 import ctypes as C
 import multiprocessing as mp
 import os
