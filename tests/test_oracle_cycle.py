@@ -177,3 +177,62 @@ def test_counters_match_published_log_line(fresh_orc):
     c = O.counters(orc, me)
     assert (c["offload_cnt"], c["release_local_cnt"], c["release_shadow_cnt"]) == \
         (g["offload"], g["releaseLocal"], g["releasePeer"])
+
+
+def test_config5_layout_four_processes(fresh_orc):
+    """benchmark configuration 5 at a quarter of its size: four simulated processes (seeds 4-7), each
+    owning the first 64 regions of configuration 2's layout, exporting every one of them and importing
+    all 192 regions of the other three. Coordinated pause and resume; every importer then reads the
+    owner's bytes at its original address. Counter closed forms from amem_nccl.cpp:511 (offload per
+    local region), :524 (releasePeer per import), :547-550 (releaseLocal per recorded importer)."""
+    orc = fresh_orc
+    live0 = orc.oracle_vmm_live_bytes()
+    P, N = 4, 64
+    fps = [Footprint(2, 4 + p, max_regions=N, threads=4) for p in range(P)]
+    own = [make_local(orc, p, fps[p]) for p in range(P)]
+    imports = {p: [] for p in range(P)}                      # importer -> (owner, region index, address)
+    for o in range(P):
+        for i, (va, h, asz) in enumerate(own[o]):
+            fd = C.c_int()
+            assert orc.oracle_vmm_export(h, C.byref(fd)) == 0
+            for q in range(P):
+                if q == o:
+                    continue
+                pva, ph = C.c_uint64(), C.c_uint64()
+                assert orc.oracle_vmm_import(fd.value, asz, C.byref(pva), C.byref(ph)) == 0
+                assert orc.oracle_add_alloc_info(q, pva.value, asz, PEER, 0, ph.value, o, h, 0, 7) == 0
+                imports[q].append((o, i, pva.value))
+            os.close(fd.value)
+    total = sum(fp.total_bytes for fp in fps)
+    # the stand-in counts what every handle holds: one handle per owner and one per import
+    assert orc.oracle_vmm_live_bytes() - live0 == P * total
+    for p in range(P):
+        assert len(O.region_table(orc, p)) == N + 3 * N
+        t = O.region_table(orc, p)[own[p][0][0]]
+        assert t["has_peer"] == 1 and sum(1 for x in t["peers"] if x) == 3
+    # everybody pauses; memory is only gone once the last importer has let go
+    for p in range(P):
+        assert orc.oracle_mem_pause(p) == 0
+        c = O.counters(orc, p)
+        assert (c["offload_cnt"], c["release_shadow_cnt"], c["release_local_cnt"]) == (N, 3 * N, 3 * N)
+    assert orc.oracle_vmm_live_bytes() == live0
+    # an importer that resumes before its owners has to wait (amem_nccl.cpp:659-662) ...
+    assert orc.oracle_mem_resume(3) == 2
+    # ... owners re-create and re-export in any order; each resume serves the importers on record
+    for p in (1, 0, 2):
+        rc = orc.oracle_mem_resume(p)
+        assert rc in (0, 2)                                   # 2 while some of p's own imports still wait
+    for p in range(P):
+        assert orc.oracle_mem_resume(p) == 0                  # idempotent once complete
+        c = O.counters(orc, p)
+        assert (c["offload_cnt"], c["release_shadow_cnt"], c["release_local_cnt"], c["paused"]) == (0, 0, 0, 0)
+    assert orc.oracle_vmm_live_bytes() - live0 == P * total
+    for p in range(P):
+        for i, (va, h, asz) in enumerate(own[p]):
+            assert fps[p].check_region(i, view(va, int(fps[p].sizes[i]))) == 0
+        for o, i, pva in imports[p]:
+            assert fps[o].check_region(i, view(pva, int(fps[o].sizes[i]))) == 0
+    view(own[2][5][0], 8)[:] = 0xC3                           # still shared memory behind all four addresses
+    for q in (0, 1, 3):
+        pva = [a for (o, i, a) in imports[q] if o == 2 and i == 5][0]
+        assert (view(pva, 8) == 0xC3).all()
