@@ -212,6 +212,10 @@ def main():
                                                 / 1e9 / d2h.value, 4),
                  "resume_copy_phase_frac": round(parked / (statistics.median(s["resume_copy_ms"] for s in stats) * 1e-3)
                                                  / 1e9 / h2d.value, 4)},
+        "unmap": {"regions": len(fp.sizes), "us_each_p50": round(statistics.median(s["pause_unmap_ms"] for s in stats)
+                                                                   * 1e3 / max(len(fp.sizes), 1), 1),
+                  "what": "time the unmapping thread spends per region (hipMemUnmap beside the gather kernel); "
+                          "the sum bounds the pause"},
         "phases_ms_p50": {k: round(statistics.median(s[k] for s in stats), 3) for k in (
             "pause_scan_ms", "pause_plan_ms", "pause_copy_ms", "pause_unmap_ms", "resume_map_ms", "resume_copy_ms",
             "k1_ms", "k2_ms", "k3_ms")},
