@@ -275,7 +275,8 @@ int amem_set_enabled(int on);
  *   "pause_xcds"      XCDs those workgroups are confined to (1-8); 0 (default) = chosen per pause
  *   "dma_min_bytes"   extents at least this long use hipMemcpyAsync in the direct path
  *   "staging_bytes"   size of each of the two device staging buffers
- *   "slab_bytes"      size of one pinned host slab (power of two)
+ *   "slab_bytes"      size of one pinned host slab (power of two, default 256 MiB); read when the
+ *                     device's engine is created, i.e. set it before the first tracked allocation
  *   "link_wgs"        workgroups of a kernel that reads or writes host memory (default 96)
  *   "hbm_wgs"         most workgroups of a kernel that touches device memory only (default 65536)
  *   "resume_batch_bytes" resume maps regions in batches of about this many bytes and follows each
