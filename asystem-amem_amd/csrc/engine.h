@@ -22,8 +22,8 @@ struct Options {
   int64_t zero_elide = 1;
   int64_t verify = 0;
   int64_t pause_path = 2;                 // 0 direct, 1 staged, 2 default (= 3), 3 interleaved, 4 reference structure (A/B only)
-  int64_t pause_wgs = 0;                  // interleaved path: workgroups of the gather kernel, 0 = chosen per pause
-  int64_t pause_xcds = 0;                 // interleaved path: XCDs the gather kernel may occupy, 0 = chosen per pause
+  int64_t pause_wgs = 0;                  // interleaved path: workgroups of the gather kernel, 0 = the default (8)
+  int64_t pause_xcds = 0;                 // interleaved path: XCDs the gather kernel may occupy, 0 = the default (1)
   int64_t interleave_bytes = 4ll << 20;   // interleaved path: parked bytes per gather launch
   int64_t dma_min_bytes = 16ll << 20;     // direct path: runs this long go by hipMemcpyAsync
   int64_t staging_bytes = 256ll << 20;    // each of two device staging buffers

@@ -270,9 +270,8 @@ int amem_set_enabled(int on);
  *                     4 = measurement aid: the reference's own structure in HIP calls (one waited-for
  *                         whole-region hipMemcpyAsync per region each way, no scan, no elision)
  *   "interleave_bytes" parked bytes per launch of path 3 (default 4 MiB)
- *   "pause_wgs"       workgroups of path 3's pack kernel; 0 (default) = chosen per pause from the
- *                     parked bytes and the number of regions
- *   "pause_xcds"      XCDs those workgroups are confined to (1-8); 0 (default) = chosen per pause
+ *   "pause_wgs"       workgroups of path 3's pack kernel; 0 (default) = 8
+ *   "pause_xcds"      XCDs those workgroups are confined to (1-8); 0 (default) = 1
  *   "dma_min_bytes"   extents at least this long use hipMemcpyAsync in the direct path
  *   "staging_bytes"   size of each of the two device staging buffers
  *   "slab_bytes"      size of one pinned host slab (power of two, default 256 MiB); read when the
