@@ -89,14 +89,19 @@ hipError_t Engine::init() {
   if (e != hipSuccess) return e;
   // Non-blocking streams at the default priority: the null stream (on which the runtime
   // runs map/unmap commands) must not wait for copies in flight.
-  e = CHECK_HIP(hipStreamCreateWithFlags(&kstream_, hipStreamNonBlocking));
-  if (e != hipSuccess) return e;
-  e = CHECK_HIP(hipStreamCreateWithFlags(&dstream_, hipStreamNonBlocking));
-  if (e != hipSuccess) return e;
+  // (a failed attempt may have left one of the streams behind: each is created once)
+  if (!kstream_) {
+    e = CHECK_HIP(hipStreamCreateWithFlags(&kstream_, hipStreamNonBlocking));
+    if (e != hipSuccess) { kstream_ = nullptr; return e; }
+  }
+  if (!dstream_) {
+    e = CHECK_HIP(hipStreamCreateWithFlags(&dstream_, hipStreamNonBlocking));
+    if (e != hipSuccess) { dstream_ = nullptr; return e; }
+  }
   // Load the kernels' code now: at the first pause there may be no device memory left for it.
   e = CHECK_HIP(preload_kernels());
   if (e != hipSuccess) return e;
-  pool_ = new SlabPool((uint64_t)options().slab_bytes);
+  if (!pool_) pool_ = new SlabPool((uint64_t)options().slab_bytes);
   inited_ = true;
   return hipSuccess;
 }
