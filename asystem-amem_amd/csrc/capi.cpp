@@ -251,7 +251,9 @@ int amem_del_alloc_info(uint64_t va, uint64_t handle, int caller) {
     if (r.tags < AMEM_MAX_CALLER) c->allocBytes[r.tags] -= r.allocSz;
     else c->delBytes += r.allocSz;
     if (handle == 0) handle = r.handle;
-    if (c->paused && c->engine) c->engine->forget(va);
+    if (c->paused) {
+      if (Engine* en = engine_if_exists(dev)) en->forget(va);  // its parked bytes are dropped
+    }
     table.erase(it);
     LOGGER(DEBUG, "groupID:%d pid:%d curDev:%d erase dptr:%llx done", amem_groupID, getpid(), dev,
            (unsigned long long)va);
@@ -437,7 +439,6 @@ int amem_mem_pause(int pid, uint64_t tag) {
     c->paused = false;
     return (int)hipErrorNoDevice;
   }
-  c->engine = en;
   bool rolled_back = false;
   int ret = en->pause(*c, &rolled_back);
   if (rolled_back) {
@@ -463,7 +464,6 @@ int amem_mem_resume(int pid, uint64_t tag) {
   if (!c->allocTable[dev].empty()) {
     Engine* en = engine_for(dev);
     if (!en) return (int)hipErrorNoDevice;
-    c->engine = en;
     bool incomplete = false;
     ret = en->resume(*c, &incomplete);
     if (incomplete) return ret;  // still paused: a later resume picks up the remaining regions

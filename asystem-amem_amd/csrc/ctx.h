@@ -17,8 +17,6 @@
 
 namespace amem {
 
-class Engine;
-class PeerService;
 
 // One tracked region, keyed by its virtual address. Field names follow the reference.
 struct Region {
@@ -68,7 +66,6 @@ struct Ctx {
   size_t pauseCnt = 0;
   size_t resumeCnt = 0;
 
-  Engine* engine = nullptr;  // created at the first pause on a machine with a GPU
 };
 
 // Global switches set at load (amem_nccl.cpp:706-723) or through the C ABI.
