@@ -377,9 +377,11 @@ int amem_check_paused(int warn) {
   Ctx* c = ctx_or_null();
   if (!c) return 0;
   std::lock_guard<std::mutex> lf(c->fields);
-  if (warn && c->paused)
+  if (warn && c->paused) {
     LOGGER(ERROR, "groupID:%d pid:%d NCCL of current process is already paused! DO NOT issue any NCCL op!",
            amem_groupID, getpid());
+    log_backtrace();  // who issued it (amem_nccl.cpp:461)
+  }
   return c->paused ? 1 : 0;
 }
 

@@ -1,6 +1,8 @@
 #include "log.h"
 
+#include <execinfo.h>
 #include <stdarg.h>
+#include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -32,6 +34,20 @@ void log_line(int level, const char* file, const char* func, int line, const cha
   std::lock_guard<std::mutex> lk(g_log_mtx);
   fprintf(stdout, "AMEM %s %s:%s:%d %s\n", tag[level], base, func, line, msg);
   if (level <= WARN) fflush(stdout);
+}
+
+// The call stack of the caller, in the layout of the reference's gtrace() (gmm_util.h:47-59).
+void log_backtrace() {
+  void* frames[96];
+  const int n = backtrace(frames, 96);
+  char** names = backtrace_symbols(frames, n);
+  if (!names) return;
+  std::lock_guard<std::mutex> lk(g_log_mtx);
+  printf("------------------\n");
+  for (int i = 0; i < n; ++i) printf("[%d] %s\n", i, names[i]);
+  printf("------------------\n");
+  fflush(stdout);
+  free(names);
 }
 
 }  // namespace amem

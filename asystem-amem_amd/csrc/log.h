@@ -14,6 +14,8 @@ int log_level();
 void set_log_level_from_env();
 void log_line(int level, const char* file, const char* func, int line, const char* fmt, ...)
     __attribute__((format(printf, 5, 6)));
+// Prints the caller's stack the way the reference's gtrace() does (gmm_util.h:47-59).
+void log_backtrace();
 
 }  // namespace amem
 

@@ -694,3 +694,23 @@ def test_wrong_handles_and_foreign_memory_at_registration(eng):
     assert lib.amem_mem_pause(0, 0) == 0 and lib.amem_mem_resume(0, 0) == 0     # with the foreign entry gone: clean
     assert regs.mismatched_bytes() == 0
     regs.free()
+
+
+def test_paused_gate_names_the_caller(eng, capfd):
+    """amem_check_paused(warn) while paused logs the reference's error line and the caller's stack
+    (amem_nccl.cpp:459-462, gtrace in gmm_util.h:47-59); without warn, or when not paused, it stays quiet."""
+    lib = eng
+    fp = Footprint(2, 41, max_regions=2, threads=2)
+    regs = H.Regions(lib, fp)
+    assert lib.amem_check_paused(1) == 0
+    assert lib.amem_mem_pause(0, 0) == 0
+    capfd.readouterr()
+    assert lib.amem_check_paused(0) == 1
+    assert "DO NOT issue" not in capfd.readouterr().out
+    assert lib.amem_check_paused(1) == 1
+    out = capfd.readouterr().out
+    assert "NCCL of current process is already paused! DO NOT issue any NCCL op!" in out
+    assert "------------------" in out and "[0] " in out and "amem_check_paused" in out
+    assert lib.amem_mem_resume(0, 0) == 0
+    assert regs.mismatched_bytes() == 0
+    regs.free()
