@@ -52,7 +52,7 @@ def cpu_baseline(threads_all, gib):
         orc.oracle_mem_pause_mt(0, threads)  # warm cycle: host buffers are created here
         orc.oracle_mem_resume_mt(0, threads)
         times = []
-        for _ in range(3):
+        for _ in range(5):
             t0 = time.perf_counter()
             orc.oracle_mem_pause_mt(0, threads)
             orc.oracle_mem_resume_mt(0, threads)
@@ -67,7 +67,7 @@ def cpu_baseline(threads_all, gib):
     assert bad == 0, "oracle cycle is not bit-exact"
     return {"value": round(out[1], 3), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": "the same footprint as the GPU run (config 3 prefix, %d regions, %.2f GiB) in the oracle's "
-                      "host-memory VMM stand-in, p50 of 3 cycles after a warm one" % (len(fp.sizes), fp.total_bytes / 2**30),
+                      "host-memory VMM stand-in, p50 of 5 cycles after a warm one" % (len(fp.sizes), fp.total_bytes / 2**30),
             "all_cores": {"value": round(out[threads_all], 3), "cores": threads_all}}
 
 
