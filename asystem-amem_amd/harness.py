@@ -149,3 +149,20 @@ def compare_tables(before, after):
         if b["type"] <= B.TYPE_LOCAL_SYMM and b["handle_gen"] != a["handle_gen"] + 1:
             diffs.append((hex(va), "handle_gen", a["handle_gen"], b["handle_gen"]))
     return diffs
+
+
+def nonzero_runs(fp, vas):
+    """Pack descriptors of a footprint as it stands: one {va, off, bytes} per run of non-zero 64 KiB
+    chunks of each region, offsets consecutive in region order. Returns (array[n, 3] uint64, bytes)."""
+    from .footprint import CHUNK
+    rows, off = [], 0
+    for i, va in enumerate(vas):
+        c0, c1 = int(fp.first_chunk[i]), int(fp.first_chunk[i + 1])
+        live = (fp.mask[c0:c1] == 0).astype(np.int8)
+        edges = np.flatnonzero(np.diff(np.concatenate([[0], live, [0]])))
+        size = int(fp.sizes[i])
+        for a, b in zip(edges[0::2], edges[1::2]):
+            start, end = int(a) * CHUNK, min(int(b) * CHUNK, size)
+            rows.append((int(va) + start, off, end - start))
+            off += end - start
+    return np.array(rows, dtype=np.uint64).reshape(-1, 3), off

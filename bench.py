@@ -156,6 +156,29 @@ def main():
                       "what": "amem_memPause/amem_memResume loop structure of the reference (amem_nccl.cpp:502-558, "
                               ":604-630) written with hipMemcpyAsync + sync per region on this GPU; p50 of 5 cycles"}
 
+    # The pack and unpack kernels on their own against the HBM roofline: the footprint's non-zero runs
+    # gathered into one device buffer and scattered back (S read + S written each way), through the C ABI.
+    hbm_kernels = None
+    descs, S = H.nonzero_runs(fp, regs.va)
+    sva, sh, sasz = C.c_uint64(), C.c_uint64(), C.c_uint64()
+    if S and lib.amem_vmm_alloc(S, 0, C.byref(sva), C.byref(sh), C.byref(sasz)) == 0:
+        dptr = descs.ctypes.data_as(C.POINTER(B.CopyDesc))
+        gms, sms, ms = [], [], C.c_float()
+        for _ in range(4):
+            assert lib.amem_gather_pack(dptr, len(descs), C.c_void_p(sva.value), S, 0, C.byref(ms)) == 0
+            gms.append(ms.value)
+            assert lib.amem_scatter_unpack(dptr, len(descs), C.c_void_p(sva.value), S, 0, C.byref(ms)) == 0
+            sms.append(ms.value)
+        lib.amem_vmm_free(sva.value, sasz.value, sh.value)
+        g, s_ = statistics.median(gms[1:]), statistics.median(sms[1:])
+        hbm_kernels = {"packed_bytes": S, "descriptors": len(descs),
+                       "gather_pack": {"ms": round(g, 3), "GBps": round(2 * S / g / 1e6, 1),
+                                       "frac_of_hbm_peak": round(2 * S / g / 1e6 / HBM_PEAK_GBPS, 4)},
+                       "scatter_unpack": {"ms": round(s_, 3), "GBps": round(2 * S / s_ / 1e6, 1),
+                                          "frac_of_hbm_peak": round(2 * S / s_ / 1e6 / HBM_PEAK_GBPS, 4)},
+                       "what": "move_tiles with a device-side buffer: 2*S bytes (S read + S written) per launch, "
+                               "p50 of 3 launches after a warm one; the bytes are checked afterwards with the rest"}
+
     # correctness gate, outside the clock: bytes, addresses, table
     bad = regs.mismatched_bytes()
     same_va = bool((regs.va == va_before).all())
@@ -220,6 +243,8 @@ def main():
             "pause_scan_ms", "pause_plan_ms", "pause_copy_ms", "pause_unmap_ms", "resume_map_ms", "resume_copy_ms",
             "k1_ms", "k2_ms", "k3_ms")},
     }
+    if hbm_kernels:
+        out["pack_unpack_in_hbm"] = hbm_kernels
     if ref_struct:
         out["reference_structure_on_gpu"] = ref_struct
         out["speedup_vs_reference_structure"] = round(out["value"] / ref_struct["value"], 3)
