@@ -79,6 +79,7 @@ def main():
     ap.add_argument("--gib", type=float, default=10.0, help="footprint budget in GiB (headline: 10)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-reference-structure", action="store_true")
+    ap.add_argument("--no-hbm-kernels", action="store_true", help="skip the pack/unpack-in-HBM measurement")
     ap.add_argument("--pause-path", type=int, default=None)
     ap.add_argument("--opt", action="append", default=[], help="engine tunable, name=value (see amem_set_option)")
     ap.add_argument("--calib", action="store_true",
@@ -161,7 +162,7 @@ def main():
     hbm_kernels = None
     descs, S = H.nonzero_runs(fp, regs.va)
     sva, sh, sasz = C.c_uint64(), C.c_uint64(), C.c_uint64()
-    if S and lib.amem_vmm_alloc(S, 0, C.byref(sva), C.byref(sh), C.byref(sasz)) == 0:
+    if S and not args.no_hbm_kernels and lib.amem_vmm_alloc(S, 0, C.byref(sva), C.byref(sh), C.byref(sasz)) == 0:
         dptr = descs.ctypes.data_as(C.POINTER(B.CopyDesc))
         gms, sms, ms = [], [], C.c_float()
         for _ in range(4):
