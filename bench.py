@@ -11,7 +11,11 @@ Prints one JSON line:
   value      2 * F / (t_pause + t_resume), GB/s (1e9), F = registered footprint bytes
   roofline   the on-device scan kernel (zero flags + checksums) against HBM peak
   link       each leg against the measured hipMemcpy rate of the host link
-  cpu_baseline  the reference's serial per-region memcpy path (oracle/) on this box's host cores
+  unmap      what the unmapping thread spends per region (the sum bounds the pause)
+  pack_unpack_in_hbm  the pack and unpack kernels with both sides in HBM, against HBM peak
+  reference_structure_on_gpu  the reference's loop structure in HIP calls on the same footprint
+  cpu_baseline  the reference's serial per-region memcpy path (oracle/) on this box's host cores,
+                same footprint
 """
 import argparse
 import ctypes as C
