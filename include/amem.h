@@ -43,16 +43,26 @@ enum amem_alloc_state {
   AMEM_STATE_MAX = 6
 };
 
-/* amem_nccl.h:52-64. type <= LOCAL_SYMM means the region owns its bytes. */
+/* amem_nccl.h:52-64. type <= LOCAL_SYMM means the region owns its bytes. Every value has two
+ * spellings: the reference's own (AMEM_TYPE_CUMEM_*, which its hook sites use) and a shorter
+ * one without the CUDA driver's prefix. */
 enum amem_alloc_type {
-  AMEM_TYPE_LOCAL = 0,
-  AMEM_TYPE_LOCAL_POSIX = 0,
-  AMEM_TYPE_LOCAL_FABRIC = 1,
-  AMEM_TYPE_LOCAL_SYMM = 2,
-  AMEM_TYPE_PEER_POSIX = 3,
-  AMEM_TYPE_PEER_FABRIC = 4,
-  AMEM_TYPE_PEER_SYMM = 5,
-  AMEM_TYPE_MAX = 6
+  AMEM_TYPE_CUMEM_LOCAL = 0,
+  AMEM_TYPE_CUMEM_LOCAL_POSIX = 0,
+  AMEM_TYPE_CUMEM_LOCAL_FABRIC = 1,
+  AMEM_TYPE_CUMEM_LOCAL_SYMM = 2,
+  AMEM_TYPE_CUMEM_PEER_POSIX = 3,
+  AMEM_TYPE_CUMEM_PEER_FABRIC = 4,
+  AMEM_TYPE_CUMEM_PEER_SYMM = 5,
+  AMEM_TYPE_CUMEM_MAX = 6,
+  AMEM_TYPE_LOCAL = AMEM_TYPE_CUMEM_LOCAL,
+  AMEM_TYPE_LOCAL_POSIX = AMEM_TYPE_CUMEM_LOCAL_POSIX,
+  AMEM_TYPE_LOCAL_FABRIC = AMEM_TYPE_CUMEM_LOCAL_FABRIC,
+  AMEM_TYPE_LOCAL_SYMM = AMEM_TYPE_CUMEM_LOCAL_SYMM,
+  AMEM_TYPE_PEER_POSIX = AMEM_TYPE_CUMEM_PEER_POSIX,
+  AMEM_TYPE_PEER_FABRIC = AMEM_TYPE_CUMEM_PEER_FABRIC,
+  AMEM_TYPE_PEER_SYMM = AMEM_TYPE_CUMEM_PEER_SYMM,
+  AMEM_TYPE_MAX = AMEM_TYPE_CUMEM_MAX
 };
 
 /* amem_nccl.h:67-80 */

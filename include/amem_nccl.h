@@ -22,7 +22,22 @@
 typedef unsigned long long amem_dptr_t;   /* CUdeviceptr in the reference */
 typedef unsigned long long amem_handle_t; /* CUmemGenericAllocationHandle in the reference */
 
-/* amem_nccl_plugin/amem_nccl.h:67-80; values equal enum amem_caller of amem.h. */
+/* amem_nccl_plugin/amem_nccl.h:39-49: AMEM_STATE_INVALID, _ALLOC, _OFFLOADING, _HOLE, _PRELOADING,
+ * _REMAPPED, _MAX with the reference's values; the enumerators live in amem.h. */
+typedef enum amem_alloc_state amem_allocState;
+
+/* amem_nccl_plugin/amem_nccl.h:52-64: AMEM_TYPE_CUMEM_LOCAL (= _LOCAL_POSIX = 0), _LOCAL_FABRIC 1,
+ * _LOCAL_SYMM 2, _PEER_POSIX 3, _PEER_FABRIC 4, _PEER_SYMM 5, _MAX 6; the enumerators live in
+ * amem.h, which is why the hook sites of the patched NCCL compile against this header as written. */
+typedef enum amem_alloc_type amem_allocType;
+
+/* amem_nccl_plugin/amem_nccl.h:82-84 */
+static inline int amem_fromPeer(amem_allocType type) {
+  return (type <= AMEM_TYPE_CUMEM_LOCAL_SYMM) ? 0 : 1;
+}
+
+/* amem_nccl_plugin/amem_nccl.h:67-80; values equal enum amem_caller of amem.h, which also holds
+ * AMEM_CALLER_MAX. */
 typedef enum {
   AMEM_CALLER_NCCL_DEFAULT = 0,
   AMEM_CALLER_NCCL_P2P = 1,

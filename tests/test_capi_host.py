@@ -38,7 +38,7 @@ def test_library_exports_every_declared_symbol(lib):
     # the reference's C++-linkage names, exactly as its library exports them
     for m in B.MANGLED_REFERENCE_SYMBOLS:
         assert m in syms, m
-    for name in declared_c_functions("amem_nccl.h"):
+    for name in declared_c_functions("amem_nccl.h") - {"amem_fromPeer"}:   # static inline in the reference's header too
         assert any(name in s and s.startswith("_Z") for s in syms), name
     # nothing internal leaks out
     leaked = [s for s in syms if s.startswith("_ZN4amem") and "scan_chunks" not in s and "calib_copy" not in s
@@ -240,14 +240,16 @@ def test_headers_compile_and_link_from_c_and_cxx(tmp_path):
     inc, libdir = os.path.join(ROOT, "include"), os.path.dirname(B.LIB_PATH)
     env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="1", AMEM_IPC="0", LD_LIBRARY_PATH=libdir + ":" + os.environ.get("LD_LIBRARY_PATH", ""))
     for compiler, std, src, exe in (("gcc", "-std=c99", "c_caller.c", "c_caller"),
-                                    ("g++", "-std=c++17", "cxx_reference_caller.cpp", "cxx_caller")):
+                                    ("g++", "-std=c++17", "cxx_reference_caller.cpp", "cxx_caller"),
+                                    # the patched NCCL's own call lines, verbatim (nccl_patch/nccl_2.27.5-1.diff)
+                                    ("g++", "-std=c++17", "cxx_hook_sites.cpp", "cxx_hook_sites")):
         out = str(tmp_path / exe)
         subprocess.run([compiler, std, "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", inc,
                         os.path.join(ROOT, "tests", "link_check", src), "-o", out, B.LIB_PATH,
                         "-Wl,-rpath," + libdir], check=True, capture_output=True, text=True)
         r = subprocess.run([out], env=env, capture_output=True, text=True, timeout=60)
         assert r.returncode == 0, (r.returncode, r.stdout[-2000:], r.stderr[-2000:])
-        assert "caller ok" in r.stdout
+        assert "caller ok" in r.stdout or "hook sites ok" in r.stdout
 
 
 def test_rccl_hook_library_exports_the_interposed_calls():
