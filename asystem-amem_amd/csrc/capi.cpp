@@ -787,6 +787,10 @@ static void __attribute__((constructor)) amem_lib_init(void) {
   amem_groupID = getenv("AMEM_GROUPID") ? atoi(getenv("AMEM_GROUPID")) : 0;
   int cuMemFlag = getenv("NCCL_CUMEM_ENABLE") ? atoi(getenv("NCCL_CUMEM_ENABLE")) : 1;
   if (cuMemFlag == 0) g.disabled = 1;
+  // The reference parses the tag (amem_nccl.cpp:478, :587) and then compares against a macro, so
+  // the variable never acts there; here it selects the caller tag whose regions are released
+  // without being copied, which is what its README documents (README.md:224, run.sh:9-18).
+  if (g.offload_free_tag >= 0 && g.offload_free_tag < AMEM_MAX_CALLER) options().offload_free_tag = g.offload_free_tag;
   LOGGER(INFO, "groupID:%d pid:%d build:%s %s NCCL plugin loaded. pause func:%s offload_free_tag:%d cuMemEnabled:%d",
          amem_groupID, getpid(), __DATE__, __TIME__, g.disabled ? "Off" : "On", g.offload_free_tag, cuMemFlag);
 }

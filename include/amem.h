@@ -294,8 +294,9 @@ int amem_set_enabled(int on);
  *   "offload_free_tag" caller tag (0-15, -1 = none) whose regions hold scratch data: pause releases
  *                     them without copying and resume hands them back zero-filled. This is what
  *                     AMEM_NCCL_OFFLOAD_FREE_TAG is documented to do in the reference, where the
- *                     variable is parsed but never takes effect (amem_nccl.cpp:40, :503, :620);
- *                     the environment variable stays ineffective here too, only this option acts
+ *                     variable is parsed but never takes effect (amem_nccl.cpp:40, :503, :620).
+ *                     Here the variable, read when the library is loaded, is this option's
+ *                     initial value
  *   "release_thread"  0/1 (default 1): the default pause path releases handles on a thread of their own
  *                     instead of on the one that unmaps
  *   "scratch_on_host" 0/1: keep the engine's own tables in pinned host memory. That is where they go

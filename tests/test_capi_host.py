@@ -5,6 +5,7 @@ import ctypes as C
 import os
 import re
 import subprocess
+import sys
 
 import numpy as np
 import pytest
@@ -328,3 +329,19 @@ def test_random_registry_sequences_match_oracle(fresh, fresh_orc, seed):
         if step % 50 == 49:
             p.check()
     p.check()
+
+
+def test_offload_free_tag_variable_becomes_the_option():
+    """AMEM_NCCL_OFFLOAD_FREE_TAG is read once, when the library is loaded (amem_nccl.cpp:478 reads it
+    per pause and never applies it); a valid tag becomes the engine's offload_free_tag option, anything
+    else leaves it off. run.sh of the reference sets 7."""
+    code = ("import sys; sys.path.insert(0, %r)\n"
+            "from asystem_amem_amd import binding as B\n"
+            "print('tag', B.load().amem_get_option(b'offload_free_tag'))\n" % ROOT)
+    for value, want in (("7", 7), ("0", 0), ("15", 15), ("16", -1), ("-3", -1), (None, -1)):
+        env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="1", AMEM_IPC="0")
+        env.pop("AMEM_NCCL_OFFLOAD_FREE_TAG", None)
+        if value is not None:
+            env["AMEM_NCCL_OFFLOAD_FREE_TAG"] = value
+        out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, check=True).stdout
+        assert ("tag %d" % want) in out, (value, out)

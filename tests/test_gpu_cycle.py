@@ -271,6 +271,7 @@ def test_offload_free_tag_releases_without_copy(eng):
     AMEM_NCCL_OFFLOAD_FREE_TAG, README.md:224, but never applies it)."""
     lib = eng
     assert lib.amem_set_option(b"offload_free_tag", B.CALLER_PROXY) == 0
+    assert lib.amem_set_option(b"verify", 1) == 0    # scratch regions are left out of the checksum comparison
     try:
         rng = np.random.default_rng(21)
         items = []
@@ -285,6 +286,7 @@ def test_offload_free_tag_releases_without_copy(eng):
         st = H.cycle_stats(lib)
         assert st["parked_bytes"] == 8 * MiB and st["footprint_bytes"] == 12 * MiB and st["zero_chunks"] == 0
         assert lib.amem_mem_resume(0, 0) == 0
+        assert H.cycle_stats(lib)["verify_mismatch"] == 0
         for va, asz, data, caller in items:
             out = np.empty(4 * MiB, dtype=np.uint8)
             lib.amem_copy_from_device(out.ctypes.data, va, out.nbytes)
@@ -294,6 +296,54 @@ def test_offload_free_tag_releases_without_copy(eng):
     finally:
         lib.amem_mem_resume(0, 0)
         assert lib.amem_set_option(b"offload_free_tag", -1) == 0
+
+
+_ENV_TAG_CHILD = r"""
+import ctypes as C, sys
+import numpy as np
+sys.path.insert(0, %r)
+from asystem_amem_amd import binding as B, harness as H
+lib = B.load()
+MiB = 1 << 20
+assert lib.amem_get_option(b"offload_free_tag") == 9, lib.amem_get_option(b"offload_free_tag")
+assert lib.amem_set_option(b"verify", 1) == 0
+rng = np.random.default_rng(33)
+items = []
+for caller in (B.CALLER_P2P, B.CALLER_PROXY, B.CALLER_POSIX, B.CALLER_PROXY):
+    va, h, asz = C.c_uint64(), C.c_uint64(), C.c_uint64()
+    assert lib.amem_vmm_alloc(6 * MiB, 0, C.byref(va), C.byref(h), C.byref(asz)) == 0
+    data = rng.integers(1, 256, 6 * MiB, dtype=np.uint8)
+    assert lib.amem_copy_to_device(va.value, data.ctypes.data, data.nbytes) == 0
+    assert lib.amem_add_alloc_info(va.value, asz.value, 0, 0, h.value, -1, 0, None, caller) == 0
+    items.append((va.value, asz.value, data, caller))
+free0 = H.mem_free(lib)
+assert lib.ncclPause(None) == 0
+st = H.cycle_stats(lib)
+assert st["footprint_bytes"] == 24 * MiB and st["parked_bytes"] == 12 * MiB, st
+assert H.mem_free(lib) - free0 >= 20 * MiB
+assert lib.ncclResume(None) == 0
+assert H.cycle_stats(lib)["verify_mismatch"] == 0 and H.counters(lib)["paused"] == 0
+for va, asz, data, caller in items:
+    out = np.empty(6 * MiB, dtype=np.uint8)
+    assert lib.amem_copy_from_device(out.ctypes.data, va, out.nbytes) == 0
+    assert (not out.any()) if caller == B.CALLER_PROXY else np.array_equal(out, data)
+    lib.amem_del_alloc_info(va, 0, 0)
+    lib.amem_vmm_free(va, asz, 0)
+print("env tag ok")
+"""
+
+
+def test_offload_free_tag_from_the_environment(gpu):
+    """Only the environment is set, the way the reference's run.sh sets it (run.sh:9-18): a process loaded
+    with AMEM_NCCL_OFFLOAD_FREE_TAG=9 parks nothing for regions registered by caller 9, releases them
+    like the others and hands them back zero-filled; regions of other callers are bit-exact."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="3", AMEM_IPC="0", AMEM_NCCL_OFFLOAD_FREE_TAG="9")
+    r = subprocess.run([sys.executable, "-c", _ENV_TAG_CHILD % root], env=env, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and "env tag ok" in r.stdout, (r.returncode, r.stdout[-3000:], r.stderr[-3000:])
+    assert "offload_free_tag:9" in r.stdout      # the load line reports what was read, as the reference's does
 
 
 def test_stale_registration_is_reported_not_read(eng):
