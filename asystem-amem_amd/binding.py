@@ -15,6 +15,8 @@ MAX_DEVS = 8
 MAX_CALLER = 16
 CHUNK = 65536
 DESC_ZERO = (1 << 64) - 1
+NOALLOC_MAX_EXTENTS = 8192
+NOALLOC_MAX_CHUNKS = 262144
 
 STATE_INVALID, STATE_ALLOC, STATE_OFFLOADING, STATE_HOLE, STATE_PRELOADING, STATE_REMAPPED = range(6)
 TYPE_LOCAL, TYPE_LOCAL_FABRIC, TYPE_LOCAL_SYMM, TYPE_PEER_POSIX, TYPE_PEER_FABRIC, TYPE_PEER_SYMM = range(6)
@@ -114,6 +116,7 @@ _SIGNATURES = {
     "amem_get_slot": (C.c_int, []),
     "amem_chunk_count": (C.c_uint64, [C.POINTER(Extent), C.c_uint64]),
     "amem_zero_scan": (C.c_int, [C.POINTER(Extent), C.c_uint64, C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
+    "amem_zero_scan_noalloc": (C.c_int, [C.POINTER(Extent), C.c_uint64, C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
     "amem_gather_pack": (C.c_int, [C.POINTER(CopyDesc), C.c_uint64, C.c_void_p, C.c_uint64, C.c_int,
                                    C.POINTER(C.c_float)]),
     "amem_scatter_unpack": (C.c_int, [C.POINTER(CopyDesc), C.c_uint64, C.c_void_p, C.c_uint64, C.c_int,

@@ -704,6 +704,13 @@ int amem_zero_scan(const amem_extent* extents, uint64_t n, uint8_t* flags, amem_
   if (!en) return (int)hipErrorNoDevice;
   return (int)en->zero_scan(extents, n, flags, sums, kernel_ms);
 }
+int amem_zero_scan_noalloc(const amem_extent* extents, uint64_t n, uint8_t* flags, amem_chunk_sum* sums,
+                           float* kernel_ms) {
+  if (int e = need_gpu("amem_zero_scan_noalloc")) return e;
+  Engine* en = engine_for(current_device());  // creates the device's engine on the first call only
+  if (!en) return (int)hipErrorNoDevice;
+  return (int)en->zero_scan_noalloc(extents, n, flags, sums, kernel_ms);
+}
 int amem_gather_pack(const amem_copy_desc* descs, uint64_t n, void* staging, uint64_t staging_bytes, int host_side,
                      float* kernel_ms) {
   if (int e = need_gpu("amem_gather_pack")) return e;

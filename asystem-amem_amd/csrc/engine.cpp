@@ -68,6 +68,10 @@ void PinBuf::release() {
   cap = 0;
 }
 
+// Pinned host staging of the allocation-free scan: segment table + chunk prefix in, flags + checksums out.
+static constexpr size_t kNaInBytes = kNoAllocMaxExtents * sizeof(ScanSeg) + (kNoAllocMaxExtents + 1) * sizeof(uint64_t);
+static constexpr size_t kNaOutBytes = kNoAllocMaxChunks * (sizeof(ChunkSum) + 1);
+
 Engine::Engine(int dev) : dev_(dev) {}
 
 Engine::~Engine() {
@@ -76,8 +80,9 @@ Engine::~Engine() {
                   &d_staging_[0], &d_staging_[1]};
   for (DevBuf* b : db) b->release();
   PinBuf* pb[] = {&h_segs_, &h_prefix_, &h_flags_, &h_sums_, &h_descs_, &h_tiles_, &h_slabtab_,
-                  &h_sums_verify_};
+                  &h_sums_verify_, &na_in_, &na_out_};
   for (PinBuf* b : pb) b->release();
+  for (hipEvent_t e : na_ev_) if (e) (void)hipEventDestroy(e);
   delete pool_;
   if (kstream_) (void)hipStreamDestroy(kstream_);
   if (dstream_) (void)hipStreamDestroy(dstream_);
@@ -102,6 +107,18 @@ hipError_t Engine::init() {
   e = CHECK_HIP(preload_kernels());
   if (e != hipSuccess) return e;
   if (!pool_) pool_ = new SlabPool((uint64_t)options().slab_bytes);
+  // Everything the allocation-free scan will ever need is made here, once per device: the device
+  // address of its fixed table array, pinned host staging for tables and results, two events.
+  if (!na_ready_) {
+    hipError_t en = CHECK_HIP(noalloc_setup(dev_));
+    if (en == hipSuccess) en = na_in_.ensure(kNaInBytes);
+    if (en == hipSuccess) en = na_out_.ensure(kNaOutBytes);
+    for (int k = 0; k < 2 && en == hipSuccess; ++k)
+      if (!na_ev_[k]) en = CHECK_HIP(hipEventCreate(&na_ev_[k]));
+    na_ready_ = (en == hipSuccess);
+    if (!na_ready_) LOGGER(WARN, "pid:%d GPU:%d set-up of the allocation-free scan failed (%d); amem_zero_scan_noalloc "
+                           "will report it", getpid(), dev_, (int)en);
+  }
   inited_ = true;
   return hipSuccess;
 }
@@ -216,6 +233,54 @@ hipError_t Engine::zero_scan(const amem_extent* ext, uint64_t n, uint8_t* flags,
     e = CHECK_HIP(hipMemcpy(sums, d_sums_.p, total * sizeof(ChunkSum), hipMemcpyDefault));
   }
   return e;
+}
+
+// Same contract and results as zero_scan. After init() has run once on this device, a call makes
+// no allocation of any kind: the tables the kernel reads and writes are the fixed device array of
+// kernels.hip, the host side of every transfer is pinned memory made by init(), the events exist.
+// Calls on one GPU share that array and the staging; busy_ is held from the first write to the last
+// read, so overlapping calls queue up instead of racing.
+hipError_t Engine::zero_scan_noalloc(const amem_extent* ext, uint64_t n, uint8_t* flags, amem_chunk_sum* sums,
+                                     float* ms) {
+  std::lock_guard<std::mutex> busy(busy_);
+  hipError_t e = init();
+  if (e != hipSuccess) return e;
+  if (!na_ready_) return hipErrorNotInitialized;
+  if (ms) *ms = 0;
+  if (n > kNoAllocMaxExtents) {
+    LOGGER(ERROR, "amem_zero_scan_noalloc: %llu extents, the fixed tables hold at most %u (use amem_zero_scan)",
+           (unsigned long long)n, kNoAllocMaxExtents);
+    return hipErrorInvalidValue;
+  }
+  ScanSeg* segs = (ScanSeg*)na_in_.p;
+  uint64_t* prefix = (uint64_t*)((uint8_t*)na_in_.p + kNoAllocMaxExtents * sizeof(ScanSeg));
+  uint64_t hint[2] = {0, 0};
+  uint64_t total = 0;
+  for (uint64_t i = 0; i < n; ++i) {
+    if ((ext[i].va & 15) || (ext[i].bytes & 15) || ext[i].va == 0) return hipErrorInvalidValue;
+    if (!inside_known_memory(ext[i].va, ext[i].bytes, hint)) return hipErrorInvalidValue;
+    segs[i] = {ext[i].va, ext[i].bytes};
+    prefix[i] = total;
+    total += chunks_of(ext[i].bytes);
+  }
+  prefix[n] = total;
+  if (total > kNoAllocMaxChunks) {
+    LOGGER(ERROR, "amem_zero_scan_noalloc: %llu chunks of 64 KiB, the fixed tables hold at most %llu (use amem_zero_scan)",
+           (unsigned long long)total, (unsigned long long)kNoAllocMaxChunks);
+    return hipErrorInvalidValue;
+  }
+  if (total == 0) return hipSuccess;
+  uint8_t* h_flags = (uint8_t*)na_out_.p + kNoAllocMaxChunks * sizeof(ChunkSum);
+  ChunkSum* h_sums = (ChunkSum*)na_out_.p;
+  e = CHECK_HIP(noalloc_scan(dev_, segs, prefix, (uint32_t)n, total, h_flags, sums ? h_sums : nullptr,
+                             (uint32_t)options().hbm_wgs, kstream_, na_ev_[0], na_ev_[1]));
+  hipError_t es = CHECK_HIP(hipStreamSynchronize(kstream_));  // also after a failed enqueue: the staging must be quiet
+  if (e != hipSuccess) return e;
+  if (es != hipSuccess) return es;
+  memcpy(flags, h_flags, total);
+  if (sums) memcpy(sums, h_sums, total * sizeof(ChunkSum));
+  if (ms) (void)CHECK_HIP(hipEventElapsedTime(ms, na_ev_[0], na_ev_[1]));
+  return hipSuccess;
 }
 
 // ---------------------------------------------------------------------------------------

@@ -88,6 +88,11 @@ class Engine {
   // Standalone kernel entry points (synchronous).
   hipError_t zero_scan(const amem_extent* ext, uint64_t n, uint8_t* flags, amem_chunk_sum* sums,
                        float* ms);
+  // zero_scan with every table in the fixed device array of kernels.hip and in pinned host
+  // buffers made by init(): allocates nothing. Rejects more than kNoAllocMaxExtents extents or
+  // kNoAllocMaxChunks chunks.
+  hipError_t zero_scan_noalloc(const amem_extent* ext, uint64_t n, uint8_t* flags, amem_chunk_sum* sums,
+                               float* ms);
   hipError_t move(bool scatter, const amem_copy_desc* descs, uint64_t n, void* staging,
                   uint64_t staging_bytes, bool host_side, float* ms);
   hipError_t probe_link(uint64_t bytes, int reps, double* d2h, double* h2d);
@@ -122,6 +127,10 @@ class Engine {
   DevBuf d_staging_[2];
   PinBuf h_segs_, h_prefix_, h_flags_, h_sums_, h_descs_, h_tiles_, h_slabtab_, h_sums_verify_;
   std::vector<hipEvent_t> events_;
+  // zero_scan_noalloc: host-side staging of the tables and results, and its own event pair
+  PinBuf na_in_, na_out_;
+  hipEvent_t na_ev_[2] = {nullptr, nullptr};
+  bool na_ready_ = false;
 
   // state carried from pause to resume
   std::vector<ParkedRegion> parked_;

@@ -3,6 +3,7 @@
 #define AMEM_KERNELS_H_
 
 #include <hip/hip_runtime_api.h>
+#include <stddef.h>
 #include <stdint.h>
 
 namespace amem {
@@ -45,6 +46,18 @@ hipError_t launch_move(bool scatter, const CopyDesc* d_descs, const uint64_t* d_
                        uint32_t ndescs, uint64_t first_tile, uint64_t ntiles,
                        const SlabTable& slabs, uint64_t off_base, uint32_t max_blocks, uint32_t xcds,
                        hipStream_t stream);
+
+// Limits of the scan that allocates nothing: its tables live in one fixed device array.
+static constexpr uint32_t kNoAllocMaxExtents = 8192;
+static constexpr uint64_t kNoAllocMaxChunks = 262144;  // 16 GiB of 64 KiB chunks
+static constexpr size_t kNoAllocScratchBytes = 131072 + 65792 + 262144 + 4194304;  // tables, each rounded to 256 B
+// Look up the device address of the fixed array for `dev`, which must be the current device. Once per device.
+hipError_t noalloc_setup(int dev);
+// Enqueue table upload, scan and result download on `stream`, using only the fixed array and the
+// caller's pinned host buffers. hipErrorInvalidValue beyond the limits above.
+hipError_t noalloc_scan(int dev, const ScanSeg* h_segs, const uint64_t* h_prefix, uint32_t nsegs,
+                        uint64_t nchunks, uint8_t* h_flags, ChunkSum* h_sums, uint32_t max_blocks,
+                        hipStream_t stream, hipEvent_t before, hipEvent_t after);
 
 // Makes the runtime load this library's device code now rather than at the first launch.
 hipError_t preload_kernels();

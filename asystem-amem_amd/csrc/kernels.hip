@@ -226,6 +226,71 @@ hipError_t launch_move(bool scatter, const CopyDesc* d_descs, const uint64_t* d_
   return hipGetLastError();
 }
 
+// ------------------------------------------------------------------------------------
+// Scan without allocation. The scan needs device memory beyond its inputs and outputs: the
+// segment table, the chunk prefix, and the flag and checksum arrays the kernel writes before
+// they are copied to the host. The ordinary path keeps those in growable hipMalloc buffers;
+// callers that may not allocate (code under graph capture, tight serving loops, harnesses that
+// forbid it) use this fixed array instead. Every GPU the library runs on holds its own copy of
+// the array, at its own address, until the process ends.
+// ------------------------------------------------------------------------------------
+
+static constexpr size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+static constexpr size_t kNaSegsOff = 0;
+static constexpr size_t kNaPrefixOff = kNaSegsOff + align256(kNoAllocMaxExtents * sizeof(ScanSeg));
+static constexpr size_t kNaFlagsOff = kNaPrefixOff + align256((kNoAllocMaxExtents + 1) * sizeof(uint64_t));
+static constexpr size_t kNaSumsOff = kNaFlagsOff + align256(kNoAllocMaxChunks);
+static constexpr size_t kNaBytes = kNaSumsOff + align256(kNoAllocMaxChunks * sizeof(ChunkSum));
+static_assert(kNaBytes == kNoAllocScratchBytes, "kernels.h states the size of the fixed scratch array");
+
+static __device__ __align__(256) uint8_t scratch[kNaBytes];
+
+// Device address of `scratch` on each GPU. In host code the array's name is only a stand-in for
+// the symbol, not an address the GPU can use: the address comes from hipGetSymbolAddress, once per
+// device, and everything below uses that pointer.
+static uint8_t* g_scratch_ptr[8] = {nullptr};
+
+hipError_t noalloc_setup(int dev) {
+  if (dev < 0 || dev >= 8) return hipErrorInvalidDevice;
+  if (g_scratch_ptr[dev]) return hipSuccess;
+  uint8_t* ptr = nullptr;
+  hipError_t e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));  // the current device's copy
+  if (e != hipSuccess) return e;
+  if (!ptr) return hipErrorInvalidSymbol;
+  g_scratch_ptr[dev] = ptr;
+  return hipSuccess;
+}
+
+// Segment table and chunk prefix come from `h_segs` / `h_prefix` (pinned host memory), the flags
+// and checksums go to `h_flags` / `h_sums` (pinned host memory; h_sums may be null). Everything is
+// enqueued on `stream`; the caller synchronises. The kernel writes entry c of both arrays for every
+// c < nchunks and only those are copied back, so nothing of an earlier call's contents is read and
+// nothing has to be cleared.
+hipError_t noalloc_scan(int dev, const ScanSeg* h_segs, const uint64_t* h_prefix, uint32_t nsegs,
+                        uint64_t nchunks, uint8_t* h_flags, ChunkSum* h_sums, uint32_t max_blocks,
+                        hipStream_t stream, hipEvent_t before, hipEvent_t after) {
+  if (dev < 0 || dev >= 8 || !g_scratch_ptr[dev]) return hipErrorNotInitialized;
+  if (nsegs == 0 || nchunks == 0) return hipSuccess;
+  if (nsegs > kNoAllocMaxExtents || nchunks > kNoAllocMaxChunks) return hipErrorInvalidValue;
+  uint8_t* ptr = g_scratch_ptr[dev];
+  ScanSeg* d_segs = (ScanSeg*)(ptr + kNaSegsOff);
+  uint64_t* d_prefix = (uint64_t*)(ptr + kNaPrefixOff);
+  uint8_t* d_flags = ptr + kNaFlagsOff;
+  ChunkSum* d_sums = (ChunkSum*)(ptr + kNaSumsOff);
+  hipError_t e = hipMemcpyAsync(d_segs, h_segs, nsegs * sizeof(ScanSeg), hipMemcpyHostToDevice, stream);
+  if (e != hipSuccess) return e;
+  e = hipMemcpyAsync(d_prefix, h_prefix, (nsegs + 1) * sizeof(uint64_t), hipMemcpyHostToDevice, stream);
+  if (e != hipSuccess) return e;
+  if (before && (e = hipEventRecord(before, stream)) != hipSuccess) return e;
+  e = launch_scan(d_segs, d_prefix, nsegs, nchunks, d_flags, h_sums ? d_sums : nullptr, max_blocks, stream);
+  if (e != hipSuccess) return e;
+  if (after && (e = hipEventRecord(after, stream)) != hipSuccess) return e;
+  e = hipMemcpyAsync(h_flags, d_flags, nchunks, hipMemcpyDeviceToHost, stream);
+  if (e != hipSuccess) return e;
+  if (h_sums) e = hipMemcpyAsync(h_sums, d_sums, nchunks * sizeof(ChunkSum), hipMemcpyDeviceToHost, stream);
+  return e;
+}
+
 hipError_t preload_kernels() {
   const void* fns[] = {(const void*)scan_chunks, (const void*)move_tiles<0>, (const void*)move_tiles<1>,
                        (const void*)calib_copy};

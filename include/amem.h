@@ -352,6 +352,24 @@ uint64_t amem_chunk_count(const amem_extent* extents, uint64_t n);
 int amem_zero_scan(const amem_extent* extents, uint64_t n, uint8_t* flags,
                    amem_chunk_sum* sums, float* kernel_ms);
 
+/* amem_zero_scan for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid it). No counterpart in the reference. Same arguments
+ * and bit-identical results; the tables the scan kernel needs beyond its inputs and outputs
+ * (segment table, chunk prefix, flags and checksums before they reach the host) live in one fixed
+ * device array of about 4.4 MiB that every GPU the library runs on holds until the process ends,
+ * and the host side of every transfer is pinned memory made when the device's engine is set up
+ * (by the first tracked allocation, or by the first call of any entry point of this section on
+ * that device). After that set-up a call allocates and frees nothing, on the device or the host.
+ * Limits: at most AMEM_NOALLOC_MAX_EXTENTS extents and AMEM_NOALLOC_MAX_CHUNKS chunks (16 GiB)
+ * per call; beyond them the call logs the limit and returns hipErrorInvalidValue (1) without
+ * touching the GPU. All calls on one GPU share the fixed array, which keeps the last call's
+ * contents; a call never reads what it has not just written, and calls that overlap on one GPU
+ * are queued on the engine's lock rather than racing. */
+#define AMEM_NOALLOC_MAX_EXTENTS 8192u
+#define AMEM_NOALLOC_MAX_CHUNKS 262144u
+int amem_zero_scan_noalloc(const amem_extent* extents, uint64_t n, uint8_t* flags,
+                           amem_chunk_sum* sums, float* kernel_ms);
+
 typedef struct amem_copy_desc {
   uint64_t va;      /* scattered side: device address, 16-byte aligned */
   uint64_t off;     /* contiguous side: byte offset into the staging buffer, 16-byte aligned;
