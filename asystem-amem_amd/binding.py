@@ -114,6 +114,8 @@ _SIGNATURES = {
     "amem_shutdown": (C.c_int, []),
     "amem_ipc_start": (C.c_int, []),
     "amem_get_slot": (C.c_int, []),
+    "amem_ipc_claim_slot": (C.c_int, []),
+    "amem_ipc_act_as": (C.c_int, [C.c_int]),
     "amem_chunk_count": (C.c_uint64, [C.POINTER(Extent), C.c_uint64]),
     "amem_zero_scan": (C.c_int, [C.POINTER(Extent), C.c_uint64, C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
     "amem_zero_scan_noalloc": (C.c_int, [C.POINTER(Extent), C.c_uint64, C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),

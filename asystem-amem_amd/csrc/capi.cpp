@@ -690,6 +690,11 @@ int amem_ipc_start(void) {
   return ipc_start(current_device());
 }
 int amem_get_slot(void) { return ipc_slot(); }
+int amem_ipc_claim_slot(void) {
+  if (ipc_slot() < 0 && ipc_start(current_device()) < 0) return -1;
+  return ipc_claim_extra();
+}
+int amem_ipc_act_as(int slot) { return ipc_act_as(slot); }
 
 // ---- kernels on their own ----
 

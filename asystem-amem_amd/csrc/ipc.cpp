@@ -47,8 +47,8 @@ struct WireReq {
 };
 static constexpr uint32_t kMagic = 0x414d454d;  // "AMEM"
 
+// One claimed slot: its lock file, its listening socket and the thread that serves it.
 struct Service {
-  std::mutex mtx;  // guards everything below except `stop`
   int slot = -1;
   int dev = 0;
   int lock_fd = -1;
@@ -57,12 +57,34 @@ struct Service {
   std::string sock_path, lock_path;
   std::thread thr;
   std::atomic<bool> stop{false};
-  int conn[AMEM_MAX_DEVS];
-  std::mutex conn_mtx[AMEM_MAX_DEVS];
-  Service() { for (int& c : conn) c = -1; }
 };
-// Never destroyed: the service thread may outlive static destruction at exit.
-Service& g_svc = *new Service();
+// A process normally holds one slot (`primary`). It may claim more, one per rank it hosts: each
+// extra slot is a full peer with a lock, a socket and a service thread of its own, so that ranks
+// living in one process reach each other exactly as ranks in different processes do.
+struct Ipc {
+  std::mutex mtx;  // guards primary / extra (not the services' own `stop`)
+  Service primary;
+  std::vector<Service*> extra;
+  int conn[AMEM_MAX_DEVS];              // client connections, by target slot
+  std::mutex conn_mtx[AMEM_MAX_DEVS];
+  Ipc() { for (int& c : conn) c = -1; }
+};
+// Never destroyed: a service thread may outlive static destruction at exit.
+Ipc& g_ipc = *new Ipc();
+Service& g_svc = g_ipc.primary;
+// The slot on whose behalf this thread registers imported regions; -1 = the primary slot.
+thread_local int t_acting_slot = -1;
+
+// Whether `slot` is one of this process's own (callers need not hold g_ipc.mtx: slots are only
+// added while no peer traffic of theirs exists, and read as plain ints).
+bool own_slot(int slot) {
+  if (slot < 0) return false;
+  if (g_svc.slot == slot) return true;
+  std::lock_guard<std::mutex> lk(g_ipc.mtx);
+  for (Service* s : g_ipc.extra) if (s->slot == slot) return true;
+  return false;
+}
+int acting_slot() { return t_acting_slot >= 0 ? t_acting_slot : g_svc.slot; }
 
 std::string ipc_dir() {
   const char* d = getenv("GMM_IPC_DIR");  // gmm_server_impl.cpp:78-79
@@ -150,7 +172,8 @@ int handle_request(const WireReq& req, int fd) {
   }
 }
 
-void serve() {
+void serve(Service* svc_p) {
+  Service& g_svc = *svc_p;
   if (gpu_present()) (void)hipSetDevice(g_svc.dev);
   std::vector<struct pollfd> fds;
   fds.push_back({g_svc.listen_fd, POLLIN, 0});
@@ -197,10 +220,12 @@ void serve() {
   for (size_t i = 2; i < fds.size(); ++i) close(fds[i].fd);
 }
 
-bool claim(int slot) {
+bool claim(int slot, Service& g_svc) {
   std::string lp = lock_name(slot);
   for (int attempt = 0; attempt < 4; ++attempt) {
-    int fd = open(lp.c_str(), O_CREAT | O_RDWR | O_CLOEXEC, 0666);
+    // Only this user's processes form a group (the service refuses everybody else), so nobody
+    // else needs to open the lock, and nobody else should be able to hold it and fake a live peer.
+    int fd = open(lp.c_str(), O_CREAT | O_RDWR | O_CLOEXEC, 0600);
     if (fd < 0) return false;
     if (flock(fd, LOCK_EX | LOCK_NB) != 0) { close(fd); return false; }
     // The lock is on the file, not on its name: if the name was removed or replaced between the
@@ -231,7 +256,7 @@ bool slot_claimed(int slot) {
 // Connect to the service of `slot`, waiting for it to appear (connect_if_not,
 // gmm_client_impl.cpp:288-347, with a bounded wait instead of an abort).
 int connect_if_not(int slot) {
-  if (g_svc.conn[slot] >= 0) return g_svc.conn[slot];
+  if (g_ipc.conn[slot] >= 0) return g_ipc.conn[slot];
   int64_t budget_ms = options().peer_timeout_ms > 0 ? options().peer_timeout_ms : 30000;
   std::string path = sock_name(slot);
   struct sockaddr_un addr = {};
@@ -241,12 +266,22 @@ int connect_if_not(int slot) {
     int s = socket(AF_UNIX, SOCK_STREAM | SOCK_CLOEXEC, 0);
     if (s < 0) return -1;
     if (connect(s, (struct sockaddr*)&addr, sizeof(addr)) == 0) {
+      // Requests carry descriptors of this process's device memory: whoever listens on the path
+      // must be a process of the same user, or it gets nothing.
+      struct ucred cred = {};
+      socklen_t clen = sizeof(cred);
+      if (getsockopt(s, SOL_SOCKET, SO_PEERCRED, &cred, &clen) != 0 || cred.uid != geteuid()) {
+        LOGGER(ERROR, "groupID:%d pid:%d %s is served by uid %d, not by this user; refusing to talk to it",
+               amem_groupID_value(), getpid(), path.c_str(), (int)cred.uid);
+        close(s);
+        return -1;
+      }
       if (options().peer_timeout_ms > 0) {
         struct timeval tv = {(time_t)(options().peer_timeout_ms / 1000), (suseconds_t)((options().peer_timeout_ms % 1000) * 1000)};
         setsockopt(s, SOL_SOCKET, SO_RCVTIMEO, &tv, sizeof(tv));
         setsockopt(s, SOL_SOCKET, SO_SNDTIMEO, &tv, sizeof(tv));
       }
-      g_svc.conn[slot] = s;
+      g_ipc.conn[slot] = s;
       return s;
     }
     close(s);
@@ -267,7 +302,7 @@ int connect_if_not(int slot) {
 
 int rpc(int slot, const WireReq& req, int fd) {
   if (slot < 0 || slot >= AMEM_MAX_DEVS) return 1;
-  std::lock_guard<std::mutex> lk(g_svc.conn_mtx[slot]);
+  std::lock_guard<std::mutex> lk(g_ipc.conn_mtx[slot]);
   int s = connect_if_not(slot);
   if (s < 0) return 1;
   int32_t ret = 1;
@@ -277,7 +312,7 @@ int rpc(int slot, const WireReq& req, int fd) {
     // peer gone, or no answer within the timeout: drop the connection so that the next
     // request reconnects instead of reading a stale reply
     close(s);
-    g_svc.conn[slot] = -1;
+    g_ipc.conn[slot] = -1;
     return 1;
   }
   return ret;
@@ -289,73 +324,110 @@ int ipc_slot() { return g_svc.slot; }
 
 bool peer_alive(int slot) { return slot >= 0 && slot < AMEM_MAX_DEVS && slot_claimed(slot); }
 
+// Bind and serve the slot `svc` has claimed. On failure the claim is given up.
+static bool start_service(Service& svc) {
+  svc.dev = current_device();
+  svc.sock_path = sock_name(svc.slot);
+  unlink(svc.sock_path.c_str());  // a stale file of a dead holder of this slot
+  svc.listen_fd = socket(AF_UNIX, SOCK_STREAM | SOCK_CLOEXEC, 0);
+  struct sockaddr_un addr = {};
+  addr.sun_family = AF_UNIX;
+  strncpy(addr.sun_path, svc.sock_path.c_str(), sizeof(addr.sun_path) - 1);
+  if (svc.listen_fd < 0 || bind(svc.listen_fd, (struct sockaddr*)&addr, sizeof(addr)) != 0 ||
+      listen(svc.listen_fd, 64) != 0 || pipe2(svc.wake, O_CLOEXEC) != 0) {
+    LOGGER(ERROR, "pid:%d failed to serve on %s error:%s", getpid(), svc.sock_path.c_str(), strerror(errno));
+    if (svc.listen_fd >= 0) close(svc.listen_fd);
+    svc.listen_fd = -1;
+    close(svc.lock_fd);
+    svc.lock_fd = -1;
+    svc.slot = -1;
+    return false;
+  }
+  svc.stop.store(false);
+  svc.thr = std::thread(serve, &svc);
+  LOGGER(DEBUG, "groupID:%d pid:%d serving slot %d on %s", amem_groupID_value(), getpid(), svc.slot,
+         svc.sock_path.c_str());
+  return true;
+}
+
+static void stop_service(Service& svc) {
+  if (svc.slot < 0) return;
+  svc.stop.store(true);
+  char b = 1;
+  if (write(svc.wake[1], &b, 1) < 0) { /* thread is woken by close below */ }
+  if (svc.thr.joinable()) svc.thr.join();
+  close(svc.listen_fd);
+  close(svc.wake[0]);
+  close(svc.wake[1]);
+  unlink(svc.sock_path.c_str());
+  // The lock file stays: removing the name while another process is between open() and flock()
+  // on it would let two processes hold "the" lock of one slot.
+  close(svc.lock_fd);
+  svc.lock_fd = svc.listen_fd = -1;
+  svc.slot = -1;
+}
+
 int ipc_start(int preferred) {
-  std::lock_guard<std::mutex> lk(g_svc.mtx);
+  std::lock_guard<std::mutex> lk(g_ipc.mtx);
   if (g_svc.slot >= 0) return g_svc.slot;
   const char* forced = getenv("AMEM_SLOT");
   bool ok = false;
   if (forced) {
     int s = atoi(forced);
-    ok = s >= 0 && s < AMEM_MAX_DEVS && claim(s);
+    ok = s >= 0 && s < AMEM_MAX_DEVS && claim(s, g_svc);
   } else {
     if (preferred < 0 || preferred >= AMEM_MAX_DEVS) preferred = 0;
-    for (int k = 0; k < AMEM_MAX_DEVS && !ok; ++k) ok = claim((preferred + k) % AMEM_MAX_DEVS);
+    for (int k = 0; k < AMEM_MAX_DEVS && !ok; ++k) ok = claim((preferred + k) % AMEM_MAX_DEVS, g_svc);
   }
   if (!ok) {
     LOGGER(WARN, "groupID:%d pid:%d no free slot under %s; cross-process regions stay out of pause scope",
            amem_groupID_value(), getpid(), ipc_dir().c_str());
     return -1;
   }
-  g_svc.dev = current_device();
-  g_svc.sock_path = sock_name(g_svc.slot);
-  unlink(g_svc.sock_path.c_str());  // a stale file of a dead holder of this slot
-  g_svc.listen_fd = socket(AF_UNIX, SOCK_STREAM | SOCK_CLOEXEC, 0);
-  struct sockaddr_un addr = {};
-  addr.sun_family = AF_UNIX;
-  strncpy(addr.sun_path, g_svc.sock_path.c_str(), sizeof(addr.sun_path) - 1);
-  if (g_svc.listen_fd < 0 || bind(g_svc.listen_fd, (struct sockaddr*)&addr, sizeof(addr)) != 0 ||
-      listen(g_svc.listen_fd, 64) != 0 || pipe2(g_svc.wake, O_CLOEXEC) != 0) {
-    LOGGER(ERROR, "pid:%d failed to serve on %s error:%s", getpid(), g_svc.sock_path.c_str(), strerror(errno));
-    if (g_svc.listen_fd >= 0) close(g_svc.listen_fd);
-    g_svc.listen_fd = -1;
-    close(g_svc.lock_fd);
-    g_svc.lock_fd = -1;
-    g_svc.slot = -1;
-    return -1;
-  }
-  g_svc.stop.store(false);
-  g_svc.thr = std::thread(serve);
-  LOGGER(DEBUG, "groupID:%d pid:%d serving slot %d on %s", amem_groupID_value(), getpid(), g_svc.slot,
-         g_svc.sock_path.c_str());
+  if (!start_service(g_svc)) return -1;
   return g_svc.slot;
 }
 
-void ipc_stop() {
-  std::lock_guard<std::mutex> lk(g_svc.mtx);
-  if (g_svc.slot < 0) return;
-  g_svc.stop.store(true);
-  char b = 1;
-  if (write(g_svc.wake[1], &b, 1) < 0) { /* thread is woken by close below */ }
-  if (g_svc.thr.joinable()) g_svc.thr.join();
-  close(g_svc.listen_fd);
-  close(g_svc.wake[0]);
-  close(g_svc.wake[1]);
-  unlink(g_svc.sock_path.c_str());
-  for (int i = 0; i < AMEM_MAX_DEVS; ++i) {
-    std::lock_guard<std::mutex> lc(g_svc.conn_mtx[i]);
-    if (g_svc.conn[i] >= 0) close(g_svc.conn[i]);
-    g_svc.conn[i] = -1;
+// One more slot for this process: a rank of its own with lock, socket and service thread.
+int ipc_claim_extra() {
+  std::lock_guard<std::mutex> lk(g_ipc.mtx);
+  if (g_svc.slot < 0) return -1;
+  Service* svc = new Service();
+  bool ok = false;
+  for (int k = 1; k < AMEM_MAX_DEVS && !ok; ++k) ok = claim((g_svc.slot + k) % AMEM_MAX_DEVS, *svc);
+  if (!ok || !start_service(*svc)) {
+    LOGGER(WARN, "groupID:%d pid:%d no further free slot under %s", amem_groupID_value(), getpid(), ipc_dir().c_str());
+    delete svc;
+    return -1;
   }
-  // The lock file stays: removing the name while another process is between open() and flock()
-  // on it would let two processes hold "the" lock of one slot.
-  close(g_svc.lock_fd);
-  g_svc.lock_fd = g_svc.listen_fd = -1;
-  g_svc.slot = -1;
+  g_ipc.extra.push_back(svc);
+  return svc->slot;
+}
+
+int ipc_act_as(int slot) {
+  if (slot < 0) { t_acting_slot = -1; return 0; }
+  if (!own_slot(slot)) return 1;
+  t_acting_slot = slot;
+  return 0;
+}
+
+void ipc_stop() {
+  std::lock_guard<std::mutex> lk(g_ipc.mtx);
+  if (g_svc.slot < 0) return;
+  for (Service* svc : g_ipc.extra) { stop_service(*svc); delete svc; }
+  g_ipc.extra.clear();
+  t_acting_slot = -1;
+  stop_service(g_svc);
+  for (int i = 0; i < AMEM_MAX_DEVS; ++i) {
+    std::lock_guard<std::mutex> lc(g_ipc.conn_mtx[i]);
+    if (g_ipc.conn[i] >= 0) close(g_ipc.conn[i]);
+    g_ipc.conn[i] = -1;
+  }
 }
 
 int peer_register(uint64_t src_handle, uint64_t my_va, int owner_slot) {
-  if (g_svc.slot < 0 || (owner_slot == g_svc.slot && !options().peer_loopback)) return 1;
-  WireReq req = {kMagic, OP_REGISTER_PEER_INFO, g_svc.slot, (int32_t)getpid(), src_handle, my_va};
+  if (g_svc.slot < 0 || (own_slot(owner_slot) && !options().peer_loopback)) return 1;
+  WireReq req = {kMagic, OP_REGISTER_PEER_INFO, acting_slot(), (int32_t)getpid(), src_handle, my_va};
   int ret = rpc(owner_slot, req, -1);
   if (ret != 0)
     LOGGER(WARN, "groupID:%d pid:%d peer_dev:%d dptr:%llx send|recv error", amem_groupID_value(), getpid(),
@@ -364,7 +436,7 @@ int peer_register(uint64_t src_handle, uint64_t my_va, int owner_slot) {
 }
 
 int peer_update(int importer_slot, uint64_t peer_va, int fd) {
-  if (importer_slot == g_svc.slot && !options().peer_loopback) return 0;
+  if (own_slot(importer_slot) && !options().peer_loopback) return 0;
   if (g_svc.slot < 0) return 1;
   WireReq req = {kMagic, OP_UPDATE_PEER_INFO, g_svc.slot, (int32_t)getpid(), 0, peer_va};
   int ret = rpc(importer_slot, req, fd);

@@ -18,6 +18,12 @@ int amem_groupID_value();
 // Claim a slot (preferring `preferred`, or AMEM_SLOT when set), bind the service socket and
 // start the service thread. Idempotent. Returns the slot, or -1.
 int ipc_start(int preferred);
+// Claim one more slot for this process (a further rank living in it), with its own lock, socket and
+// service thread. Needs the primary service. Returns the slot, or -1.
+int ipc_claim_extra();
+// From now on this thread registers imported regions as `slot` (one of this process's own; -1 =
+// the primary slot again). 0 ok, 1 when the process does not hold that slot.
+int ipc_act_as(int slot);
 void ipc_stop();
 int ipc_slot();
 // Whether a process currently holds `slot` of this group (a crashed one no longer does).

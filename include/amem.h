@@ -328,6 +328,17 @@ int amem_shutdown(void);
  * otherwise started by the first add of a peer-type region or by amem_get_slot). */
 int amem_ipc_start(void);
 int amem_get_slot(void);
+/* A process that hosts several ranks gives each of them a slot of its own: amem_ipc_claim_slot
+ * claims one more slot for this process (lock file, socket and service thread like the first one)
+ * and returns it, or -1 when none is free. amem_ipc_act_as(slot) makes the calling thread register
+ * the imported regions it adds from then on as that slot (-1: as the process's first slot again);
+ * 0 ok, 1 when this process does not hold `slot`. With "peer_loopback" on, the ranks of one process
+ * register with and update each other over their sockets exactly as ranks in different processes
+ * do; with it off (default) they follow the reference's same-process rule and stay out of each
+ * other's pause scope (gmm_client_impl.cpp:482-484). No reference counterpart: the reference has
+ * one worker per (process, GPU). */
+int amem_ipc_claim_slot(void);
+int amem_ipc_act_as(int slot);
 
 /* ---------------------------------------------------------------------------------------
  * 6. The device kernels, callable on their own (no reference counterpart: the reference

@@ -363,3 +363,97 @@ def test_owner_forgets_an_importer_whose_process_is_gone(gpu, fresh):
     assert lib.amem_mem_resume(0, 0) == 0 and regs.mismatched_bytes() == 0
     regs.free()
 
+
+
+def test_config5_shape_three_importer_ranks_in_one_process(gpu, fresh):
+    """Benchmark configuration 5 at its full per-process shape, in the one form this machine's runtime
+    allows (it refuses a VMM descriptor exported by another process): the process holds four slots, each
+    with its own lock, socket and service thread; the first owns the 256 regions of configuration 2's
+    layout (1,216 MiB), each of the other three imports all 256 at addresses of its own. 768 registration
+    requests, and per resume 768 descriptor messages (SCM_RIGHTS) to three different services, each of
+    which maps the new memory at its importer's original address. Counter closed forms as for the oracle's
+    tests/test_oracle_cycle.py::test_config5_layout_four_processes (amem_nccl.cpp:511 offload per local
+    region, :524 releasePeer per import, :547-550 releaseLocal per recorded importer)."""
+    from asystem_amem_amd import binding as B, harness as H
+    from asystem_amem_amd.footprint import Footprint
+    lib = fresh
+    assert lib.amem_set_option(b"peer_loopback", 1) == 0
+    try:
+        N, R = 256, 3
+        fp = Footprint(2, 4, max_regions=N, threads=8)
+        regs = H.Regions(lib, fp)
+        assert len(regs.va) == N and fp.total_bytes == 1216 * MiB
+        owner = lib.amem_get_slot()
+        ranks = [lib.amem_ipc_claim_slot() for _ in range(R)]
+        assert owner >= 0 and len({owner, *ranks}) == R + 1 and min(ranks) >= 0
+        imports = {}                                         # (rank slot, region) -> importer's address
+        for s in ranks:
+            assert lib.amem_ipc_act_as(s) == 0
+            for i in range(N):
+                fd, va, h = C.c_int(-1), C.c_uint64(), C.c_uint64()
+                assert lib.amem_vmm_export(int(regs.handle[i]), C.byref(fd)) == 0
+                assert lib.amem_vmm_import(fd.value, int(regs.alloc[i]), 0, C.byref(va), C.byref(h)) == 0
+                os.close(fd.value)
+                assert lib.amem_add_alloc_info(va.value, int(regs.alloc[i]), B.TYPE_PEER_POSIX, 0, h.value, owner,
+                                               int(regs.handle[i]), None, B.CALLER_P2P_PEER) == 0
+                imports[(s, i)] = va.value
+        assert lib.amem_ipc_act_as(-1) == 0
+        assert len(set(imports.values())) == R * N
+
+        def imports_match():
+            bad = 0
+            buf = np.empty(int(fp.sizes.max()), dtype=np.uint8)
+            for (s, i), va in imports.items():
+                n = int(fp.sizes[i])
+                assert lib.amem_copy_from_device(buf.ctypes.data, va, n) == 0
+                bad += fp.check_region(i, buf[:n])
+            return bad
+
+        tab = H.region_table(lib, 0)
+        assert len(tab) == N + R * N
+        for i in range(N):                                   # every owner entry knows its three importers
+            t = tab[int(regs.va[i])]
+            assert t["has_peer"] == 1
+            assert {s: p for s, p in enumerate(t["peers"]) if p} == {s: imports[(s, i)] for s in ranks}
+        c = H.counters(lib)
+        assert c["alloc_bytes"][B.CALLER_P2P] == fp.total_bytes and c["alloc_bytes"][B.CALLER_P2P_PEER] == R * fp.total_bytes
+        assert imports_match() == 0
+        before = H.region_table(lib, 0)
+        assert lib.amem_mem_pause(0, 0) == 0 and lib.amem_mem_resume(0, 0) == 0     # warm cycle: engine scratch, pinned pool
+        fds0, free0 = _nfds(), H.mem_free(lib)
+        times = []
+        for cycle in range(2):
+            assert lib.amem_mem_pause(0, 0) == 0
+            c = H.counters(lib)
+            assert (c["offload_cnt"], c["release_shadow_cnt"], c["release_local_cnt"]) == (N, R * N, R * N)
+            assert H.mem_free(lib) - free0 >= fp.total_bytes - 8 * MiB   # all four references to every region are gone
+            assert all(t["state"] == B.STATE_HOLE for t in H.region_table(lib, 0).values())
+            assert lib.amem_check_paused(0) == 1
+            assert lib.amem_mem_resume(0, 0) == 0
+            st = H.cycle_stats(lib)
+            times.append((st["pause_ms"], st["resume_ms"], st["resume_peer_ms"]))
+            c = H.counters(lib)
+            assert (c["offload_cnt"], c["release_shadow_cnt"], c["release_local_cnt"], c["paused"]) == (0, 0, 0, 0)
+            assert _nfds() == fds0                           # 256 exported and 768 received descriptors, all closed
+            assert regs.mismatched_bytes() == 0              # the owner's bytes at the owner's addresses
+            assert imports_match() == 0                      # and at all 768 importer addresses
+        after = H.region_table(lib, 0)
+        assert [d for d in H.compare_tables(before, after) if d[1] != "handle_gen"] == []
+        assert all(after[va]["handle_gen"] == before[va]["handle_gen"] + 3 for va in before)   # three cycles, three new handles each
+        print("config-5 shape, one process: %d regions x %d importers, pause/resume/peer ms per cycle: %s" %
+              (N, R, ", ".join("%.0f/%.0f/%.0f" % t for t in times)))
+        # one physical memory behind all four addresses of a region
+        tag = np.full(4096, 0xC3, dtype=np.uint8)
+        assert lib.amem_copy_to_device(int(regs.va[5]), tag.ctypes.data, 4096) == 0
+        for s in ranks:
+            buf = np.empty(4096, dtype=np.uint8)
+            assert lib.amem_copy_from_device(buf.ctypes.data, imports[(s, 5)], 4096) == 0
+            assert (buf == 0xC3).all()
+        for (s, i), va in imports.items():
+            lib.amem_del_alloc_info(va, 0, 0)
+            lib.amem_vmm_free(va, int(regs.alloc[i]), 0)
+        regs.free()
+    finally:
+        lib.amem_mem_resume(0, 0)
+        lib.amem_ipc_act_as(-1)
+        assert lib.amem_set_option(b"peer_loopback", 0) == 0

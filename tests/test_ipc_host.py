@@ -118,3 +118,61 @@ def test_a_peer_that_died_is_noticed_at_once():
         i_in[1].send("exit")
         imp.join(30)
         assert imp.exitcode == 0
+
+
+def _several_ranks(ipc_dir, gid, to_parent):
+    os.environ.update(AMEM_ENABLE="1", GMM_LOG="1", GMM_IPC_DIR=ipc_dir, AMEM_GROUPID=str(gid))
+    from asystem_amem_amd import binding as B, harness as H
+    lib = B.load()
+    out = {}
+    owned = [(OWNER_VA + (k << 30), OWNER_HANDLE + k) for k in range(4)]
+    for va, h in owned:
+        assert lib.amem_add_alloc_info(va, 4 * MiB, B.TYPE_LOCAL, 0, h, -1, 0, None, B.CALLER_P2P) == 0
+    first = lib.amem_get_slot()
+    extra = [lib.amem_ipc_claim_slot() for _ in range(3)]
+    out["slots"] = [first] + extra
+    out["sockets"] = sorted(f for f in os.listdir(ipc_dir) if f.endswith(".sock"))
+    out["foreign"] = lib.amem_ipc_act_as((max(out["slots"]) + 1) % 8 if len(set(out["slots"])) < 8 else 0)
+    # same-process rule of the reference while loopback is off: a rank does not register with a rank of its own process
+    assert lib.amem_ipc_act_as(extra[0]) == 0
+    out["refused"] = lib.amem_add_alloc_info(0x7e0000000000, 4 * MiB, B.TYPE_PEER_POSIX, 0, 0x900, first, owned[0][1],
+                                             None, B.CALLER_P2P_PEER)
+    assert lib.amem_set_option(b"peer_loopback", 1) == 0
+    want = {}
+    for r, slot in enumerate(extra):
+        assert lib.amem_ipc_act_as(slot) == 0
+        for k, (va, h) in enumerate(owned):
+            my_va = 0x7e1000000000 + (r << 36) + (k << 30)
+            assert lib.amem_add_alloc_info(my_va, 4 * MiB, B.TYPE_PEER_POSIX, 0, 0x1000 + 16 * r + k, first, h, None,
+                                           B.CALLER_P2P_PEER) == 0
+            want.setdefault(va, {})[slot] = my_va
+    assert lib.amem_ipc_act_as(-1) == 0
+    tab = H.region_table(lib, 0)
+    out["table_size"] = len(tab)
+    out["peers_ok"] = all(tab[va]["has_peer"] == 1 and
+                          {s: p for s, p in enumerate(tab[va]["peers"]) if p} == want[va] for va, _ in owned)
+    assert lib.amem_set_option(b"peer_loopback", 0) == 0
+    lib.amem_shutdown()
+    out["sockets_after"] = [f for f in os.listdir(ipc_dir) if f.endswith(".sock")]
+    to_parent.send(out)
+
+
+def test_several_ranks_in_one_process_each_hold_a_slot():
+    """A process claims three more slots; each has its own lock, socket and service thread, and regions
+    imported on behalf of each of them are recorded by the owner under that slot: the layout of benchmark
+    configuration 5 (every region imported by three peers) inside one process. Registry only, no GPU."""
+    ctx = mp.get_context("spawn")
+    with tempfile.TemporaryDirectory() as ipc_dir:
+        out_r, out_w = ctx.Pipe(duplex=False)
+        p = ctx.Process(target=_several_ranks, args=(ipc_dir, 0x7000 + os.getpid() % 4096, out_w))
+        p.start()
+        assert out_r.poll(60)
+        out = out_r.recv()
+        p.join(30)
+        assert p.exitcode == 0
+        assert len(set(out["slots"])) == 4 and all(0 <= s < 8 for s in out["slots"])
+        assert len(out["sockets"]) == 4
+        assert out["foreign"] == 1                         # cannot act as a slot the process does not hold
+        assert out["refused"] == 1
+        assert out["table_size"] == 4 + 12 and out["peers_ok"]
+        assert out["sockets_after"] == []
