@@ -13,117 +13,10 @@ from multiprocessing import reduction
 import numpy as np
 import pytest
 
+from peer_worker import _nfds, run_world
+
 pytestmark = pytest.mark.gpu
 MiB = 1 << 20
-NREG = 6          # regions per process (config-2 distribution: 4 MiB channel buffers first)
-
-
-def _nfds():
-    return len(os.listdir("/proc/self/fd"))
-
-
-def _worker(rank, world, ipc_dir, gid, conns, ctrl):
-    """conns[j]: duplex connection to rank j (None for self); ctrl: connection to the parent."""
-    try:
-        os.environ.update(AMEM_ENABLE="1", GMM_LOG="2", GMM_IPC_DIR=ipc_dir, AMEM_GROUPID=str(gid), AMEM_SLOT=str(rank))
-        from asystem_amem_amd import binding as B, harness as H
-        from asystem_amem_amd.footprint import Footprint
-        lib = B.load()
-        lib.amem_set_option(b"peer_timeout_ms", 60000)
-        fp = Footprint(2, 4 + rank, max_regions=NREG, threads=2)
-        regs = H.Regions(lib, fp)                      # local regions, registered
-        assert lib.amem_get_slot() == rank
-        ctrl.send(("ready", rank)); assert ctrl.recv() == "go"
-        # export to every peer
-        for j in range(world):
-            if j == rank:
-                continue
-            for i in range(NREG):
-                fd = C.c_int(-1)
-                assert lib.amem_vmm_export(int(regs.handle[i]), C.byref(fd)) == 0
-                conns[j].send((i, int(regs.handle[i]), int(regs.alloc[i])))
-                reduction.send_handle(conns[j], fd.value, None)
-                os.close(fd.value)
-        # import from every peer and register with the owner
-        imported = {}   # (owner, i) -> (va, size)
-        for j in range(world):
-            if j == rank:
-                continue
-            for _ in range(NREG):
-                i, owner_handle, size = conns[j].recv()
-                fd = reduction.recv_handle(conns[j])
-                va, h = C.c_uint64(), C.c_uint64()
-                assert lib.amem_vmm_import(fd, size, 0, C.byref(va), C.byref(h)) == 0
-                os.close(fd)
-                rc = lib.amem_add_alloc_info(va.value, size, B.TYPE_PEER_POSIX, 0, h.value, j, owner_handle, None,
-                                             B.CALLER_P2P_PEER)
-                assert rc == 0, ("register with owner failed", rank, j, i, rc)
-                imported[(j, i)] = (va.value, size)
-        ctrl.send(("imported", rank)); assert ctrl.recv() == "go"
-        peers_fp = {j: Footprint(2, 4 + j, max_regions=NREG, threads=2) for j in range(world) if j != rank}
-
-        def check_imports():
-            bad = 0
-            for (j, i), (va, size) in imported.items():
-                n = int(peers_fp[j].sizes[i])
-                buf = np.empty(n, dtype=np.uint8)
-                assert lib.amem_copy_from_device(buf.ctypes.data, va, n) == 0
-                bad += peers_fp[j].check_region(i, buf)
-            return bad
-
-        assert check_imports() == 0
-        tab = H.region_table(lib, 0)
-        for i in range(NREG):                          # every owner entry knows all its importers
-            t = tab[int(regs.va[i])]
-            assert t["has_peer"] == 1 and sum(1 for p in t["peers"] if p) == world - 1 and t["peers"][rank] == 0
-        before = {va: dict(t) for va, t in tab.items()}
-        fds0 = _nfds()
-        free0 = H.mem_free(lib)
-        ctrl.send(("checked", rank, free0)); assert ctrl.recv() == "go"
-        for cycle in range(2):
-            assert lib.amem_mem_pause(0, 0) == 0
-            c = H.counters(lib)
-            assert (c["offload_cnt"], c["release_local_cnt"], c["release_shadow_cnt"]) == \
-                (NREG, NREG * (world - 1), NREG * (world - 1))
-            for va, t in H.region_table(lib, 0).items():
-                assert t["state"] == B.STATE_HOLE
-            ctrl.send(("paused", rank)); assert ctrl.recv() == "go"
-            freed = H.mem_free(lib) - free0            # all ranks paused: everybody's memory is gone
-            assert freed >= world * fp.total_bytes - 64 * MiB, (freed, world * fp.total_bytes)
-            ctrl.send(("freed", rank)); assert ctrl.recv() == "go"
-            if cycle == 1 and rank == 0:
-                time.sleep(0.3)                        # importers must wait for a late owner, not fail
-            assert lib.amem_mem_resume(0, 0) == 0
-            c = H.counters(lib)
-            assert (c["offload_cnt"], c["release_local_cnt"], c["release_shadow_cnt"], c["paused"]) == (0, 0, 0, 0)
-            ctrl.send(("resumed", rank)); assert ctrl.recv() == "go"
-            assert regs.mismatched_bytes() == 0        # own bytes
-            assert check_imports() == 0                # peers' bytes at this process's original VAs
-            after = H.region_table(lib, 0)
-            diffs = [d for d in H.compare_tables(before, after) if d[1] != "handle_gen"]
-            assert diffs == [], diffs
-            assert _nfds() == fds0, (fds0, _nfds())    # exported and received fds are all closed
-            ctrl.send(("verified", rank)); assert ctrl.recv() == "go"
-        # an owner's write after resume is visible through the importers' old addresses
-        if rank == 0:
-            tag = np.full(4096, 0xA7, dtype=np.uint8)
-            assert lib.amem_copy_to_device(int(regs.va[0]), tag.ctypes.data, 4096) == 0
-        ctrl.send(("tagged", rank)); assert ctrl.recv() == "go"
-        if rank != 0:
-            buf = np.empty(4096, dtype=np.uint8)
-            assert lib.amem_copy_from_device(buf.ctypes.data, imported[(0, 0)][0], 4096) == 0
-            assert (buf == 0xA7).all()
-        ctrl.send(("done", rank)); assert ctrl.recv() == "go"
-        for (j, i), (va, size) in imported.items():
-            lib.amem_del_alloc_info(va, 0, 0)
-            lib.amem_vmm_free(va, size, 0)
-        regs.free()
-        lib.amem_shutdown()
-        ctrl.send(("exit", rank))
-    except BaseException as e:  # report instead of hanging the barrier
-        import traceback
-        ctrl.send(("error", rank, traceback.format_exc()))
-        raise
 
 
 def _probe_owner(conn):
@@ -183,39 +76,7 @@ def test_processes_sharing_one_gpu(gpu, world):
         pytest.skip("this machine's HIP runtime cannot import a VMM fd exported by another process "
                     "(hipMemImportFromShareableHandle -> invalid argument); the same path is covered in one "
                     "process by test_peer_path_in_loopback and between processes on the CPU by tests/test_ipc_host.py")
-    ctx = mp.get_context("spawn")
-    with tempfile.TemporaryDirectory() as ipc_dir:
-        gid = 0x6000 + os.getpid() % 4096 + world
-        pair = {}
-        for a in range(world):
-            for b in range(a + 1, world):
-                pair[(a, b)], pair[(b, a)] = ctx.Pipe(duplex=True)
-        ctrls = [ctx.Pipe(duplex=True) for _ in range(world)]
-        procs = []
-        for r in range(world):
-            conns = [pair.get((r, j)) for j in range(world)]
-            p = ctx.Process(target=_worker, args=(r, world, ipc_dir, gid, conns, ctrls[r][1]))
-            p.start()
-            procs.append(p)
-        try:
-            phases = ["ready", "imported", "checked"] + ["paused", "freed", "resumed", "verified"] * 2 + ["tagged", "done"]
-            for phase in phases:
-                for r in range(world):
-                    assert ctrls[r][0].poll(120), "rank %d did not reach %s" % (r, phase)
-                    msg = ctrls[r][0].recv()
-                    assert msg[0] == phase, msg
-                for r in range(world):
-                    ctrls[r][0].send("go")
-            for r in range(world):
-                assert ctrls[r][0].poll(60)
-                assert ctrls[r][0].recv()[0] == "exit"
-            for p in procs:
-                p.join(60)
-                assert p.exitcode == 0
-        finally:
-            for p in procs:
-                if p.is_alive():
-                    p.kill()
+    run_world(world)
 
 
 @pytest.mark.parametrize("nregions", [5, 256])
