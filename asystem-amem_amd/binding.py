@@ -56,7 +56,8 @@ class CycleStats(C.Structure):
         (n, C.c_uint64) for n in (
         "k1_launches", "k2_launches", "k3_launches", "footprint_bytes", "parked_bytes", "zero_chunks",
         "total_chunks", "local_regions", "peer_regions", "dma_bytes", "kernel_bytes", "slab_bytes",
-        "verify_mismatch")]
+        "verify_mismatch")] + [(n, C.c_double) for n in (
+        "pause_pool_ms", "pause_scratch_ms", "pause_sync_ms", "resume_scratch_ms")]
 
     def as_dict(self):
         return {k: getattr(self, k) for k, _ in self._fields_}

@@ -613,6 +613,7 @@ static OptRef* opt_table(size_t* n) {
       {"slab_bytes", &o.slab_bytes, 1 << 16, (int64_t)1 << 36},
       {"link_wgs", &o.link_wgs, 1, 65536},
       {"hbm_wgs", &o.hbm_wgs, 1, 1 << 20},
+      {"hbm_move_wgs", &o.hbm_move_wgs, 1, (int64_t)1 << 30},
       {"resume_batch_bytes", &o.resume_batch_bytes, 1, (int64_t)1 << 40},
       {"peer_timeout_ms", &o.peer_timeout_ms, 0, (int64_t)1 << 40},
       {"peer_loopback", &o.peer_loopback, 0, 1},

@@ -25,6 +25,19 @@ Options& options() {
   return o;
 }
 
+// Host time spent allocating engine scratch (tables, staging, events) since the counter was last
+// read; pause and resume report it as a phase of their own. Only touched under Engine::busy_.
+static double g_scratch_alloc_ms = 0;
+static double take_scratch_alloc_ms() {
+  const double v = g_scratch_alloc_ms;
+  g_scratch_alloc_ms = 0;
+  return v;
+}
+struct ScratchTimer {
+  Clock::time_point t0 = Clock::now();
+  ~ScratchTimer() { g_scratch_alloc_ms += ms_since(t0); }
+};
+
 // Pause is called when device memory is short, possibly gone. Scratch that does not fit on
 // the device goes to pinned host memory, which the kernels reach over the link: slower
 // table lookups, same results.
@@ -32,6 +45,7 @@ hipError_t DevBuf::ensure(size_t bytes, bool grow_on_host) {
   const bool forced = options().scratch_on_host != 0;
   if (bytes <= cap && (!forced || host)) return hipSuccess;
   const bool want_host = forced || grow_on_host;
+  ScratchTimer timed;
   release();
   size_t want = std::max<size_t>(bytes + bytes / 4, 4096);
   if (!want_host) {
@@ -55,6 +69,7 @@ void DevBuf::release() {
 }
 hipError_t PinBuf::ensure(size_t bytes) {
   if (bytes <= cap) return hipSuccess;
+  ScratchTimer timed;
   release();
   size_t want = std::max<size_t>(bytes + bytes / 4, 4096);
   hipError_t e = CHECK_HIP(hipHostMalloc(&p, want, hipHostMallocDefault));
@@ -125,6 +140,7 @@ hipError_t Engine::init() {
 
 hipEvent_t Engine::event_at(size_t i) {
   while (events_.size() <= i) {
+    ScratchTimer timed;
     hipEvent_t ev = nullptr;
     (void)CHECK_HIP(hipEventCreate(&ev));
     events_.push_back(ev);
@@ -417,7 +433,8 @@ hipError_t Engine::move(bool scatter, const amem_copy_desc* descs, uint64_t n, v
   (void)CHECK_HIP(hipEventRecord(e0, kstream_));
   e = CHECK_HIP(launch_move(scatter, (const CopyDesc*)d_descs_.p, (const uint64_t*)d_tiles_.p,
                             (uint32_t)n, 0, ntiles, st, 0,
-                            (uint32_t)(host_side ? options().link_wgs : options().hbm_wgs), 8, kstream_));
+                            (uint32_t)(host_side ? options().link_wgs : options().hbm_move_wgs),
+                            host_side ? 8 : kXcdsHbmShape, kstream_));
   if (e != hipSuccess) return e;
   (void)CHECK_HIP(hipEventRecord(e1, kstream_));
   e = CHECK_HIP(hipStreamSynchronize(kstream_));
@@ -723,7 +740,7 @@ hipError_t Engine::pause_copy_staged(Ctx& c, std::vector<Region*>& regs, bool* u
         (void)CHECK_HIP(hipEventRecord(s0, kstream_));
         e = CHECK_HIP(launch_move(false, (const CopyDesc*)d_descs_.p + d0, (const uint64_t*)d_tiles_.p + d0,
                                   d1 - d0, tp[d0], tp[d1] - tp[d0], stg, base,
-                                  (uint32_t)options().hbm_wgs, 8, kstream_));
+                                  (uint32_t)options().hbm_move_wgs, kXcdsHbmShape, kstream_));
         if (e != hipSuccess) return e;
         (void)CHECK_HIP(hipEventRecord(s1, kstream_));
         e = CHECK_HIP(hipEventSynchronize(s1));
@@ -786,11 +803,13 @@ int Engine::pause(Ctx& c, bool* rolled_back) {
   stats_ = fresh;
 
   auto& table = c.allocTable[dev_];
+  (void)take_scratch_alloc_ms();
   note(CHECK_HIP(hipDeviceSynchronize()));
   size_t free_sz = 0, total = 0;
   (void)CHECK_HIP(hipMemGetInfo(&free_sz, &total));
   LOGGER(INFO, "memPause: groupID:%d pid:%d GPU:%d memUsed: %ld MB before paused", amem_groupID_value(),
          getpid(), dev_, (long)((total - free_sz) >> 20));
+  stats_.pause_sync_ms = ms_since(t0);
 
   std::vector<Region*> locals, invalid;
   std::vector<std::pair<uint64_t, Region*>> imported;
@@ -921,7 +940,9 @@ int Engine::pause(Ctx& c, bool* rolled_back) {
            amem_groupID_value(), getpid(), dev_, (unsigned long long)(cursor >> 20), (unsigned long long)(limit >> 20));
     e = hipErrorOutOfMemory;
   } else {
+    auto tpool = Clock::now();
     e = pool_->ensure(cursor);
+    stats_.pause_pool_ms = ms_since(tpool);
   }
   note(e);
   // Resume's scatter list is the gather list plus the zero runs (plus one entry per region that
@@ -1001,6 +1022,7 @@ int Engine::pause(Ctx& c, bool* rolled_back) {
     n_offload = c.offloadCnt; n_local = c.releaseLocalCnt; n_shadow = c.releaseShadowCnt;
   }
   stats_.pause_ms = ms_since(t0);
+  stats_.pause_scratch_ms = take_scratch_alloc_ms();
   (void)CHECK_HIP(hipMemGetInfo(&free_sz, &total));
   LOGGER(INFO, "memPause: pause results. groupID:%d pid:%d GPU:%d pauseCnt:%ld memUsed:%ld MB after paused, "
          "released:%ld MB, duration:%ld ms offload:%d releaseLocal:%d releasePeer:%d",
@@ -1038,6 +1060,7 @@ int Engine::resume(Ctx& c, bool* incomplete) {
   auto t0 = Clock::now();
   stats_.resume_ms = stats_.resume_map_ms = stats_.resume_copy_ms = stats_.resume_peer_ms = 0;
   stats_.k3_ms = 0; stats_.k3_launches = 0; stats_.verify_mismatch = 0;
+  (void)take_scratch_alloc_ms();
   auto& table = c.allocTable[dev_];
 
   // A pause that failed half-way leaves regions it never released in OFFLOADING: they still
@@ -1279,6 +1302,7 @@ int Engine::resume(Ctx& c, bool* incomplete) {
     }
   }
   stats_.resume_ms = ms_since(t0);
+  stats_.resume_scratch_ms = take_scratch_alloc_ms();
   (void)CHECK_HIP(hipMemGetInfo(&free_sz, &total));
   long n_resume;
   int n_offload, n_local, n_shadow;

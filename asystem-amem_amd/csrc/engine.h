@@ -29,7 +29,8 @@ struct Options {
   int64_t staging_bytes = 256ll << 20;    // each of two device staging buffers
   int64_t slab_bytes = 256ll << 20;
   int64_t link_wgs = 96;                  // workgroups of a kernel touching host memory
-  int64_t hbm_wgs = 65536;                // workgroup cap of device-only kernels
+  int64_t hbm_wgs = 65536;                // workgroup cap of the scan kernel
+  int64_t hbm_move_wgs = 1 << 22;         // workgroup cap of the mover when both sides are device memory
   int64_t resume_batch_bytes = 64ll << 20;
   int64_t peer_timeout_ms = 60000;
   int64_t release_thread = 1;             // interleaved path: handles are released on a third thread

@@ -42,6 +42,9 @@ hipError_t launch_scan(const ScanSeg* d_segs, const uint64_t* d_chunk_prefix, ui
                        uint64_t nchunks, uint8_t* d_flags, ChunkSum* d_sums, uint32_t max_blocks,
                        hipStream_t stream);
 
+// `xcds` = 1..8 confines the link-shaped mover to that many XCDs; kXcdsHbmShape selects the mover
+// shaped for device memory on both sides (`max_blocks` then caps its grid of 4 KiB pieces).
+static constexpr uint32_t kXcdsHbmShape = 0xffffffffu;
 hipError_t launch_move(bool scatter, const CopyDesc* d_descs, const uint64_t* d_tile_prefix,
                        uint32_t ndescs, uint64_t first_tile, uint64_t ntiles,
                        const SlabTable& slabs, uint64_t off_base, uint32_t max_blocks, uint32_t xcds,

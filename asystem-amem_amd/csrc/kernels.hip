@@ -177,6 +177,61 @@ __global__ __launch_bounds__(kBlock) void move_tiles(const CopyDesc* __restrict_
   }
 }
 
+// The same mover shaped for the case where both sides are device memory, which is bound by HBM
+// rather than by the host link. Measured on an MI355X with the benchmark footprint's 33,600 runs
+// (6.9 GiB, read + written counted): the link shape above (16 KiB per 256 lanes, 4 loads in flight
+// per lane, 65,536 workgroups striding) 5.7 TB/s; the same without striding 5.8; 8 KiB per 256
+// lanes 6.1; 4 KiB per 64 lanes 6.1; 2 KiB per 64 lanes 6.2; any shape with a single load per lane
+// 4.6; this one — 4 KiB per workgroup of two wavefronts, two 16-byte loads in flight per lane,
+// non-temporal, one workgroup per piece with no stride loop up to the grid cap — 6.4 TB/s, 80 % of
+// the HBM peak (plain loads and stores instead of non-temporal ones: 5.8). The descriptor of a
+// piece is found in the same 16 KiB tile prefix (a piece is a quarter of a tile); a direct
+// piece-to-descriptor table measured the same as the search.
+static constexpr int kHbmBlock = 128;
+static constexpr uint32_t kHbmPiece = 4096;
+static constexpr uint32_t kPiecesPerTile = (uint32_t)(kTileBytes / kHbmPiece);
+static_assert(kHbmPiece == kHbmBlock * 16 * 2, "two 16-byte loads per lane");
+
+template <int MODE>
+__global__ __launch_bounds__(kHbmBlock) void move_pieces_hbm(const CopyDesc* __restrict__ descs,
+                                                             const uint64_t* __restrict__ tile_prefix,
+                                                             uint32_t ndescs, uint64_t first_tile,
+                                                             uint64_t ntiles, SlabTable slabs,
+                                                             uint64_t off_base) {
+  const uint32_t tid = threadIdx.x;
+  const uint64_t npieces = ntiles * kPiecesPerTile;
+  for (uint64_t w = blockIdx.x; w < npieces; w += gridDim.x) {
+    const uint64_t t = first_tile + w / kPiecesPerTile;
+    const uint32_t d = find_segment(tile_prefix, ndescs, t);
+    const uint64_t o = (t - tile_prefix[d]) * kTileBytes + (w % kPiecesPerTile) * kHbmPiece;
+    const uint64_t bytes = descs[d].bytes;
+    if (o >= bytes) continue;  // the last tile of a descriptor may have fewer pieces
+    const uint64_t rem = bytes - o;
+    const uint32_t nvec = (uint32_t)(rem < kHbmPiece ? rem : kHbmPiece) >> 4;
+    const uint64_t off = descs[d].off;
+    u32x4* dev = (u32x4*)(descs[d].va + o);
+    if (MODE == 1 && off == kDescZero) {
+      const u32x4 z = {0u, 0u, 0u, 0u};
+      for (uint32_t i = tid; i < nvec; i += kHbmBlock) __builtin_nontemporal_store(z, dev + i);
+      continue;
+    }
+    u32x4* stg = (u32x4*)slab_addr(slabs, off - off_base + o);
+    const u32x4* __restrict__ src = (MODE == 0) ? dev : stg;
+    u32x4* __restrict__ dst = (MODE == 0) ? stg : dev;
+    if (nvec == kHbmPiece / 16) {
+      u32x4 a = __builtin_nontemporal_load(src + tid);
+      u32x4 b = __builtin_nontemporal_load(src + tid + kHbmBlock);
+      __builtin_nontemporal_store(a, dst + tid);
+      __builtin_nontemporal_store(b, dst + tid + kHbmBlock);
+    } else {
+      for (uint32_t i = tid; i < nvec; i += kHbmBlock) {
+        u32x4 a = __builtin_nontemporal_load(src + i);
+        __builtin_nontemporal_store(a, dst + i);
+      }
+    }
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void calib_copy(const u32x4* __restrict__ src,
                                                      u32x4* __restrict__ dst, uint64_t nvec) {
   uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -211,6 +266,19 @@ hipError_t launch_move(bool scatter, const CopyDesc* d_descs, const uint64_t* d_
                        const SlabTable& slabs, uint64_t off_base, uint32_t max_blocks, uint32_t xcds,
                        hipStream_t stream) {
   if (ntiles == 0 || ndescs == 0) return hipSuccess;
+  if (xcds == kXcdsHbmShape) {
+    // both sides in device memory: one small workgroup per 4 KiB piece
+    const uint64_t npieces = ntiles * kPiecesPerTile;
+    const uint32_t grid = (uint32_t)(npieces < max_blocks ? npieces : max_blocks);
+    (void)hipGetLastError();
+    if (scatter)
+      hipLaunchKernelGGL(move_pieces_hbm<1>, dim3(grid), dim3(kHbmBlock), 0, stream, d_descs, d_tile_prefix,
+                         ndescs, first_tile, ntiles, slabs, off_base);
+    else
+      hipLaunchKernelGGL(move_pieces_hbm<0>, dim3(grid), dim3(kHbmBlock), 0, stream, d_descs, d_tile_prefix,
+                         ndescs, first_tile, ntiles, slabs, off_base);
+    return hipGetLastError();
+  }
   if (xcds < 1 || xcds > kXcds) xcds = kXcds;
   // the grid is a multiple of 8 so that every XCD is dealt the same number of workgroups;
   // `max_blocks` counts the workgroups that actually work
@@ -293,7 +361,7 @@ hipError_t noalloc_scan(int dev, const ScanSeg* h_segs, const uint64_t* h_prefix
 
 hipError_t preload_kernels() {
   const void* fns[] = {(const void*)scan_chunks, (const void*)move_tiles<0>, (const void*)move_tiles<1>,
-                       (const void*)calib_copy};
+                       (const void*)move_pieces_hbm<0>, (const void*)move_pieces_hbm<1>, (const void*)calib_copy};
   for (const void* f : fns) {
     hipFuncAttributes attr;
     hipError_t e = hipFuncGetAttributes(&attr, f);

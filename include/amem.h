@@ -255,6 +255,10 @@ typedef struct amem_cycle_stats {
   uint64_t kernel_bytes;    /* of parked_bytes, how much moved by the pack/unpack kernels */
   uint64_t slab_bytes;      /* pinned host memory held by the pool */
   uint64_t verify_mismatch; /* chunks whose checksum differed after resume (verify mode) */
+  double pause_pool_ms;     /* of pause_ms: growing the pinned host pool (non-zero when slabs were added) */
+  double pause_scratch_ms;  /* of pause_ms: allocating or growing the engine's own tables, staging and events */
+  double pause_sync_ms;     /* of pause_ms: the device synchronisation and memory queries before the scan */
+  double resume_scratch_ms; /* of resume_ms: allocating or growing the engine's own tables and events */
 } amem_cycle_stats;
 void amem_get_cycle_stats(amem_cycle_stats* out);
 
@@ -287,7 +291,9 @@ int amem_set_enabled(int on);
  *   "slab_bytes"      size of one pinned host slab (power of two, default 256 MiB); read when the
  *                     device's engine is created, i.e. set it before the first tracked allocation
  *   "link_wgs"        workgroups of a kernel that reads or writes host memory (default 96)
- *   "hbm_wgs"         most workgroups of a kernel that touches device memory only (default 65536)
+ *   "hbm_wgs"         most workgroups of the scan kernel (default 65536)
+ *   "hbm_move_wgs"    most workgroups of the pack/unpack kernel when both sides are device memory
+ *                     (default 4194304: one workgroup per 4 KiB piece up to 16 GiB, striding beyond)
  *   "resume_batch_bytes" resume maps regions in batches of about this many bytes and follows each
  *                     batch with one unpack launch (default 64 MiB)
  *   "peer_timeout_ms" how long resume waits for owners before failing (0 = forever)

@@ -37,10 +37,11 @@ def make_local(orc, ctx, fp, caller=1):
 
 
 def test_config1_cycle_identity_table_and_release(fresh_orc):
-    """benchmark configuration 1 at a quarter of its size (16 of the 64 regions): host-memcpy pause to
-    a host buffer then restore; byte compare plus region-table compare."""
+    """benchmark configuration 1 at its full size (64 regions of 2 MiB x U{1..16}, seed 0, about 1 GiB):
+    host-memcpy pause to a host buffer then restore; byte compare plus region-table compare."""
     orc = fresh_orc
-    fp = Footprint(1, 0, max_regions=16)
+    fp = Footprint(1, 0)
+    assert len(fp.sizes) == 64
     live0 = orc.oracle_vmm_live_bytes()
     regs = make_local(orc, 0, fp)
     assert orc.oracle_vmm_live_bytes() - live0 == fp.total_bytes
@@ -49,7 +50,8 @@ def test_config1_cycle_identity_table_and_release(fresh_orc):
     # post-conditions of amem_memPause: every entry HOLE, handle 0, not in handleTable, memory gone
     c = O.counters(orc, 0)
     assert (c["paused"], c["pause_cnt"], c["offload_cnt"], c["release_local_cnt"], c["release_shadow_cnt"],
-            c["handle_count"]) == (1, 1, 16, 0, 0, 0)
+            c["handle_count"]) == (1, 1, 64, 0, 0, 0)
+    assert orc.oracle_check_paused(0) == 1                                                  # the gate, amem_nccl.cpp:452-464
     assert orc.oracle_vmm_live_bytes() == live0
     for va, t in O.region_table(orc, 0).items():
         assert t["state"] == ST_HOLE and t["handle"] == 0 and t["cpu_addr"] != 0
@@ -58,7 +60,8 @@ def test_config1_cycle_identity_table_and_release(fresh_orc):
     assert orc.oracle_mem_resume(0) == 0
     after = O.region_table(orc, 0)
     c = O.counters(orc, 0)
-    assert (c["paused"], c["resume_cnt"], c["offload_cnt"], c["handle_count"]) == (0, 1, 0, 16)
+    assert (c["paused"], c["resume_cnt"], c["offload_cnt"], c["handle_count"]) == (0, 1, 0, 64)
+    assert orc.oracle_check_paused(0) == 0
     assert orc.oracle_mem_resume(0) == 0 and O.counters(orc, 0)["resume_cnt"] == 1         # idempotent (:591-593)
     assert set(after) == set(before)
     for va in before:
