@@ -10,8 +10,22 @@
 //   hipMemMap(ptr, size, handle)   remembers the pending mapping
 //   hipMemSetAccess(ptr, size)     the mapping is now usable  -> amem_add_alloc_info(ptr, size, LOCAL, dev, handle)
 //   hipMemUnmap(ptr, size)         the mapping is going away  -> amem_del_alloc_info(ptr) first
-//   hipMemImportFromShareableHandle remembers imported handles: their mappings are another
-//                                  process's memory and are not registered by this hook
+//   hipMemExportToShareableHandle  the owner's side of an exchange: remembers which handle the exported
+//                                  descriptor stands for, under the descriptor's identity (device and inode
+//                                  numbers of the file behind it, which every duplicate of it shares), in
+//                                  this process and as a small file under GMM_IPC_DIR for other processes
+//   hipMemImportFromShareableHandle the importer's side: looks the descriptor's identity up and so learns
+//                                  the owner's slot and the owner's handle value; a later hipMemSetAccess
+//                                  on a mapping of the imported handle registers it as somebody else's
+//                                  memory -> amem_add_alloc_info(ptr, size, PEER_POSIX, dev, handle,
+//                                  owner slot, owner handle), the shape of the reference's hook in
+//                                  ncclP2pImportShareableBuffer (nccl_patch/nccl_2.27.5-1.diff:572-579).
+//                                  An import whose owner cannot be named stays unregistered.
+//
+// What interposition cannot see: the reference also takes buffers out of the registry just before
+// they are registered with a NIC (diff:309-312, :364-367, :379-488). RCCL reaches the verbs library
+// and the dma-buf export of the HSA runtime through dlopen + dlsym on explicit handles, which no
+// library placed in front of them can intercept; a patched RCCL calls amem_delAllocInfo there itself.
 //
 // Calls made by anything else (the pause/resume engine itself, the application) pass through
 // untouched. The module a call comes from is found from its return address.
@@ -20,6 +34,10 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <string>
 
 #include <mutex>
 #include <unordered_map>
@@ -41,8 +59,33 @@ struct Pending {
 std::mutex g_mtx;
 std::unordered_map<uint64_t, Pending> g_mapped;      // RCCL mappings seen at hipMemMap
 std::unordered_set<uint64_t> g_registered;           // those handed to the registry
-std::unordered_set<uint64_t> g_imported_handles;     // handles RCCL imported from a peer
+struct Owner {
+  int slot;         // slot of the owning process, -1 when unknown
+  uint64_t handle;  // the owner's handle value
+};
+std::unordered_map<uint64_t, Owner> g_imported_handles;   // handles RCCL imported from a peer -> who owns the memory
+std::unordered_map<std::string, Owner> g_exports;         // descriptor identity -> this process's handle behind it
+std::unordered_map<uint64_t, std::string> g_export_of;    // exported handle -> descriptor identity (to forget it again)
+std::unordered_map<uint64_t, std::string> g_export_at;    // address the exported handle was mapped at -> identity; the
+                                                          // handle value changes with every resume, the address never
 int g_verbose = -1;
+
+// What every duplicate of a descriptor has in common, in this and in any other process.
+std::string identity_of(int fd) {
+  struct stat st;
+  if (fd < 0 || fstat(fd, &st) != 0) return std::string();
+  char b[64];
+  snprintf(b, sizeof(b), "%llx_%llx", (unsigned long long)st.st_dev, (unsigned long long)st.st_ino);
+  return b;
+}
+std::string export_file(const std::string& id) {
+  int gid = 0;
+  amem_get_group_id(&gid);
+  const char* d = getenv("GMM_IPC_DIR");
+  char b[320];
+  snprintf(b, sizeof(b), "%s/amem_export_%x_%s", d ? d : "/tmp", gid, id.c_str());
+  return b;
+}
 
 bool verbose() {
   if (g_verbose < 0) g_verbose = getenv("AMEM_HOOK_LOG") ? atoi(getenv("AMEM_HOOK_LOG")) : 0;
@@ -101,22 +144,36 @@ HOOK_API hipError_t hipMemSetAccess(void* ptr, size_t size, const hipMemAccessDe
   hipError_t e = fn(ptr, size, desc, count);
   if (e != hipSuccess || !from_rccl(__builtin_return_address(0))) return e;
   Pending p = {0, 0};
-  bool fresh = false;
+  Owner owner = {-1, 0};
+  bool fresh = false, imported = false;
   {
     std::lock_guard<std::mutex> lk(g_mtx);
     auto it = g_mapped.find((uint64_t)(uintptr_t)ptr);
-    if (it != g_mapped.end() && !g_imported_handles.count(it->second.handle)) {
-      p = it->second;
-      fresh = g_registered.insert((uint64_t)(uintptr_t)ptr).second;
+    if (it != g_mapped.end()) {
+      auto im = g_imported_handles.find(it->second.handle);
+      if (im != g_imported_handles.end()) { imported = true; owner = im->second; }
+      if (!imported || owner.slot >= 0) {
+        p = it->second;
+        fresh = g_registered.insert((uint64_t)(uintptr_t)ptr).second;
+      } else if (verbose()) {
+        fprintf(stderr, "AMEM [DEBG] rccl_hook: %p maps an imported handle whose owner is unknown; not registered\n", ptr);
+      }
     }
   }
   if (fresh) {
     int dev = 0;
     (void)hipGetDevice(&dev);
-    // the shape of the reference's hook in ncclCuMemAlloc (nccl_patch/nccl_2.27.5-1.diff:278-280)
-    int rc = amem_add_alloc_info((uint64_t)(uintptr_t)ptr, p.size, AMEM_TYPE_LOCAL, dev, p.handle, -1, 0, NULL,
-                                 AMEM_CALLER_DEFAULT);
-    if (verbose()) fprintf(stderr, "AMEM [DEBG] rccl_hook: registered %p size %zu rc %d\n", ptr, p.size, rc);
+    int rc;
+    if (imported)
+      // the shape of the reference's hook in ncclP2pImportShareableBuffer (nccl_patch/nccl_2.27.5-1.diff:572-579)
+      rc = amem_add_alloc_info((uint64_t)(uintptr_t)ptr, p.size, AMEM_TYPE_PEER_POSIX, dev, p.handle, owner.slot,
+                               owner.handle, NULL, AMEM_CALLER_P2P_PEER);
+    else
+      // the shape of the reference's hook in ncclCuMemAlloc (nccl_patch/nccl_2.27.5-1.diff:278-280)
+      rc = amem_add_alloc_info((uint64_t)(uintptr_t)ptr, p.size, AMEM_TYPE_LOCAL, dev, p.handle, -1, 0, NULL,
+                               AMEM_CALLER_DEFAULT);
+    if (verbose()) fprintf(stderr, "AMEM [DEBG] rccl_hook: registered %p size %zu %s rc %d\n", ptr, p.size,
+                           imported ? "imported" : "local", rc);
     if (rc != 0) {
       std::lock_guard<std::mutex> lk(g_mtx);
       g_registered.erase((uint64_t)(uintptr_t)ptr);
@@ -129,11 +186,20 @@ HOOK_API hipError_t hipMemUnmap(void* ptr, size_t size) {
   static auto fn = real<hipError_t (*)(void*, size_t)>("hipMemUnmap");
   if (from_rccl(__builtin_return_address(0))) {
     bool was_registered;
+    std::string id;
     {
       std::lock_guard<std::mutex> lk(g_mtx);
       was_registered = g_registered.erase((uint64_t)(uintptr_t)ptr) > 0;
       g_mapped.erase((uint64_t)(uintptr_t)ptr);
+      auto ex = g_export_at.find((uint64_t)(uintptr_t)ptr);
+      if (ex != g_export_at.end()) {
+        id = ex->second;
+        auto ow = g_exports.find(id);
+        if (ow != g_exports.end()) { g_export_of.erase(ow->second.handle); g_exports.erase(ow); }
+        g_export_at.erase(ex);
+      }
     }
+    if (!id.empty()) unlink(export_file(id).c_str());   // the note for importers in other processes
     // the shape of the reference's hook in ncclCuMemFree (nccl_patch/nccl_2.27.5-1.diff:288-290)
     if (was_registered) (void)amem_del_alloc_info((uint64_t)(uintptr_t)ptr, 0, 0);
     if (verbose()) fprintf(stderr, "AMEM [DEBG] rccl_hook: unmap %p size %zu registered %d\n", ptr, size, (int)was_registered);
@@ -147,10 +213,81 @@ HOOK_API hipError_t hipMemImportFromShareableHandle(hipMemGenericAllocationHandl
       "hipMemImportFromShareableHandle");
   hipError_t e = fn(handle, osHandle, shHandleType);
   if (e == hipSuccess && handle && from_rccl(__builtin_return_address(0))) {
+    Owner owner = {-1, 0};
+    if (shHandleType == hipMemHandleTypePosixFileDescriptor) {
+      const std::string id = identity_of((int)(uintptr_t)osHandle);
+      bool found = false;
+      if (!id.empty()) {
+        std::lock_guard<std::mutex> lk(g_mtx);
+        auto it = g_exports.find(id);
+        if (it != g_exports.end()) { owner = it->second; found = true; }
+      }
+      if (!found && !id.empty()) {
+        // exported by another process: it left a note under the descriptor's identity
+        if (FILE* f = fopen(export_file(id).c_str(), "r")) {
+          int slot = -1;
+          unsigned long long h = 0;
+          if (fscanf(f, "%d %llx", &slot, &h) == 2) owner = {slot, (uint64_t)h};
+          fclose(f);
+        }
+      }
+    }
+    if (verbose()) fprintf(stderr, "AMEM [DEBG] rccl_hook: imported handle %p, owner slot %d handle %llx\n", (void*)*handle,
+                           owner.slot, (unsigned long long)owner.handle);
     std::lock_guard<std::mutex> lk(g_mtx);
-    g_imported_handles.insert((uint64_t)(uintptr_t)*handle);
+    g_imported_handles[(uint64_t)(uintptr_t)*handle] = owner;
   }
   return e;
+}
+
+HOOK_API hipError_t hipMemExportToShareableHandle(void* shareableHandle, hipMemGenericAllocationHandle_t handle,
+                                                  hipMemAllocationHandleType handleType, unsigned long long flags) {
+  static auto fn = real<hipError_t (*)(void*, hipMemGenericAllocationHandle_t, hipMemAllocationHandleType, unsigned long long)>(
+      "hipMemExportToShareableHandle");
+  hipError_t e = fn(shareableHandle, handle, handleType, flags);
+  if (e == hipSuccess && shareableHandle && handleType == hipMemHandleTypePosixFileDescriptor &&
+      from_rccl(__builtin_return_address(0))) {
+    const std::string id = identity_of(*(int*)shareableHandle);
+    const int slot = amem_get_slot();
+    if (!id.empty() && slot >= 0) {
+      const uint64_t h = (uint64_t)(uintptr_t)handle;
+      std::string stale;
+      {
+        std::lock_guard<std::mutex> lk(g_mtx);
+        auto old = g_export_of.find(h);
+        if (old != g_export_of.end() && old->second != id) stale = old->second;
+        g_exports[id] = {slot, h};
+        g_export_of[h] = id;
+        int dev = 0;
+        (void)hipGetDevice(&dev);
+        if (uint64_t va = amem_handle_lookup(dev, h)) g_export_at[va] = id;
+      }
+      if (!stale.empty()) unlink(export_file(stale).c_str());
+      if (FILE* f = fopen(export_file(id).c_str(), "w")) {
+        fprintf(f, "%d %llx %d\n", slot, (unsigned long long)h, (int)getpid());
+        fclose(f);
+      }
+      if (verbose()) fprintf(stderr, "AMEM [DEBG] rccl_hook: exported handle %p as %s (slot %d)\n", (void*)handle, id.c_str(), slot);
+    }
+  }
+  return e;
+}
+
+// hipMemRelease from RCCL ends a handle's life as far as RCCL is concerned: forget what was noted about it.
+HOOK_API hipError_t hipMemRelease(hipMemGenericAllocationHandle_t handle) {
+  static auto fn = real<hipError_t (*)(hipMemGenericAllocationHandle_t)>("hipMemRelease");
+  if (from_rccl(__builtin_return_address(0))) {
+    std::string id;
+    {
+      std::lock_guard<std::mutex> lk(g_mtx);
+      const uint64_t h = (uint64_t)(uintptr_t)handle;
+      g_imported_handles.erase(h);
+      auto it = g_export_of.find(h);
+      if (it != g_export_of.end()) { id = it->second; g_exports.erase(id); g_export_of.erase(it); }
+    }
+    if (!id.empty()) unlink(export_file(id).c_str());
+  }
+  return fn(handle);
 }
 
 // Number of RCCL mappings currently mirrored into the registry (for tests and diagnostics).

@@ -46,3 +46,29 @@ extern "C" __attribute__((visibility("default"))) int standin_cumem_free(void* p
   if (hipMemAddressFree(ptr, size) != hipSuccess) return 5;
   return 0;
 }
+
+// The owner's half of a buffer exchange, as ncclP2pAllocateShareableBuffer does it: the handle is
+// looked up from the address and exported as a POSIX file descriptor.
+extern "C" __attribute__((visibility("default"))) int standin_export(void* ptr, int* fd) {
+  hipMemGenericAllocationHandle_t handle = nullptr;
+  if (hipMemRetainAllocationHandle(&handle, ptr) != hipSuccess) return 1;
+  if (hipMemExportToShareableHandle((void*)fd, handle, hipMemHandleTypePosixFileDescriptor, 0) != hipSuccess) return 2;
+  return 0;
+}
+
+// The importer's half, in the call order of ncclP2pImportShareableBuffer
+// (nccl_patch/nccl_2.27.5-1.diff:560-590): import, reserve, map, allow access by the local GPU.
+extern "C" __attribute__((visibility("default"))) int standin_import_map(int fd, size_t size, void** ptr) {
+  hipMemGenericAllocationHandle_t handle = nullptr;
+  if (hipMemImportFromShareableHandle(&handle, (void*)(uintptr_t)fd, hipMemHandleTypePosixFileDescriptor) != hipSuccess) return 1;
+  if (hipMemAddressReserve(ptr, size, 0, nullptr, 0) != hipSuccess) return 2;
+  if (hipMemMap(*ptr, size, 0, handle, 0) != hipSuccess) return 3;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 4;
+  hipMemAccessDesc acc = {};
+  acc.location.type = hipMemLocationTypeDevice;
+  acc.location.id = dev;
+  acc.flags = hipMemAccessFlagsProtReadWrite;
+  if (hipMemSetAccess(*ptr, size, &acc, 1) != hipSuccess) return 5;
+  return 0;
+}

@@ -155,3 +155,102 @@ def test_real_rccl_communicator_works_across_cycles(gpu):
         (r.returncode, r.stdout[-3000:], r.stderr[-3000:])
     if "rccl skipped" in r.stdout:
         pytest.skip("librccl.so is not loadable on this machine")
+
+
+IMPORT_CHILD = r'''
+import ctypes as C, os, sys
+import numpy as np
+root, standin = sys.argv[1], sys.argv[2]
+sys.path.insert(0, root)
+libdir = os.path.join(root, "asystem-amem_amd", "lib")
+hook = C.CDLL(os.path.join(libdir, "libamem_rccl_hook.so"), mode=C.RTLD_GLOBAL)
+from asystem_amem_amd import binding as B, harness as H
+lib = B.load()
+rccl = C.CDLL(standin, mode=C.RTLD_GLOBAL)
+rccl.standin_cumem_alloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+rccl.standin_cumem_free.argtypes = [C.c_void_p]
+rccl.standin_export.argtypes = [C.c_void_p, C.POINTER(C.c_int)]
+rccl.standin_import_map.argtypes = [C.c_int, C.c_size_t, C.POINTER(C.c_void_p)]
+hook.amem_rccl_hook_registered.restype = C.c_int64
+MiB = 1 << 20
+ipc_dir = os.environ["GMM_IPC_DIR"]
+notes = lambda: sorted(f for f in os.listdir(ipc_dir) if f.startswith("amem_export_"))
+rng = np.random.default_rng(41)
+# rank A (the process's first slot) allocates the way ncclCuMemAlloc does
+owned = []
+for n in (4 * MiB, 8 * MiB, 2 * MiB):
+    p = C.c_void_p()
+    assert rccl.standin_cumem_alloc(C.byref(p), n) == 0
+    data = rng.integers(1, 256, n, dtype=np.uint8)
+    assert lib.amem_copy_to_device(p.value, data.ctypes.data, n) == 0
+    owned.append((p.value, n, data))
+slot_a = lib.amem_get_slot()
+assert slot_a >= 0 and lib.amem_region_count(0) == 3
+# without the loopback option two ranks of one process follow the reference's same-process rule:
+# the import is mapped and works, but stays outside the registry (gmm_client_impl.cpp:482-484)
+slot_b = lib.amem_ipc_claim_slot()
+assert slot_b >= 0 and slot_b != slot_a and lib.amem_ipc_act_as(slot_b) == 0
+fd, q = C.c_int(-1), C.c_void_p()
+assert rccl.standin_export(owned[2][0], C.byref(fd)) == 0
+assert rccl.standin_import_map(fd.value, owned[2][1], C.byref(q)) == 0
+os.close(fd.value)
+assert lib.amem_region_count(0) == 3 and hook.amem_rccl_hook_registered() == 3
+assert rccl.standin_cumem_free(q.value) == 0
+# with it, rank B registers what it imports with rank A through the socket service
+assert lib.amem_set_option(b"peer_loopback", 1) == 0
+imports = []
+for p, n, data in owned:
+    fd, q = C.c_int(-1), C.c_void_p()
+    assert lib.amem_ipc_act_as(-1) == 0
+    assert rccl.standin_export(p, C.byref(fd)) == 0              # rank A exports
+    assert lib.amem_ipc_act_as(slot_b) == 0
+    assert rccl.standin_import_map(fd.value, n, C.byref(q)) == 0  # rank B imports and maps
+    os.close(fd.value)
+    imports.append(q.value)
+assert lib.amem_ipc_act_as(-1) == 0
+assert len(notes()) == 3                                           # one note per exported buffer, for importers elsewhere
+tab = H.region_table(lib, 0)
+assert len(tab) == 6 and hook.amem_rccl_hook_registered() == 6
+for (p, n, _), q in zip(owned, imports):
+    assert tab[q]["type"] == B.TYPE_PEER_POSIX and tab[q]["alloc_sz"] == n and tab[q]["tags"] == B.CALLER_P2P_PEER
+    assert tab[q]["mc_handle"] == tab[p]["handle"]                 # the owner's handle value travelled with the descriptor
+    assert tab[p]["has_peer"] == 1 and tab[p]["peers"][slot_b] == q
+lib.ncclPause(None); lib.ncclResume(None)                          # warm cycle
+free0 = H.mem_free(lib)
+assert lib.ncclPause(None) == 0
+c = H.counters(lib)
+assert (c["offload_cnt"], c["release_shadow_cnt"], c["release_local_cnt"]) == (3, 3, 3)
+assert H.mem_free(lib) - free0 >= 14 * MiB - 2 * MiB              # the importer let go first, so the memory really went
+assert lib.ncclResume(None) == 0
+c = H.counters(lib)
+assert (c["offload_cnt"], c["release_shadow_cnt"], c["release_local_cnt"], c["paused"]) == (0, 0, 0, 0)
+for (p, n, data), q in zip(owned, imports):
+    for addr in (p, q):
+        out = np.empty(n, dtype=np.uint8)
+        assert lib.amem_copy_from_device(out.ctypes.data, addr, n) == 0 and np.array_equal(out, data)
+# rank B drops its mappings, then rank A frees: the registry and the notes empty out
+for q in imports:
+    assert rccl.standin_cumem_free(q) == 0
+assert lib.amem_region_count(0) == 3
+for p, n, _ in owned:
+    assert rccl.standin_cumem_free(p) == 0
+assert lib.amem_region_count(0) == 0 and hook.amem_rccl_hook_registered() == 0 and notes() == []
+print("rccl hook import side ok")
+'''
+
+
+def test_hook_registers_imported_mappings_with_their_owner(gpu, tmp_path):
+    """The importer's half of the hook (the reference's site in ncclP2pImportShareableBuffer,
+    nccl_patch/nccl_2.27.5-1.diff:572-579): a second rank, living in the same process under a slot of its
+    own, imports the descriptors the first rank exports; the hook names the owner from the descriptor's
+    identity and registers each mapping as PEER_POSIX, so a pause drops the importer's mappings before
+    the owner's release and a resume maps the new memory back at the importer's addresses."""
+    standin = str(tmp_path / "librccl_standin.so")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    subprocess.run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-D__HIP_PLATFORM_AMD__",
+                    "-I" + os.path.join(rocm, "include"), os.path.join(ROOT, "tests", "rccl_standin", "librccl_standin.cpp"),
+                    "-o", standin, "-L" + os.path.join(rocm, "lib"), "-lamdhip64"], check=True, capture_output=True, text=True)
+    env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="1", GMM_IPC_DIR=str(tmp_path), AMEM_GROUPID=str(0x7400 + os.getpid() % 1024))
+    env.pop("AMEM_IPC", None)
+    r = subprocess.run([sys.executable, "-c", IMPORT_CHILD, ROOT, standin], env=env, capture_output=True, text=True, timeout=240)
+    assert r.returncode == 0 and "rccl hook import side ok" in r.stdout, (r.returncode, r.stdout[-3000:], r.stderr[-3000:])
