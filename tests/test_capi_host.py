@@ -43,7 +43,7 @@ def test_library_exports_every_declared_symbol(lib):
         assert any(name in s and s.startswith("_Z") for s in syms), name
     # nothing internal leaks out
     leaked = [s for s in syms if s.startswith("_ZN4amem") and "scan_chunks" not in s and "calib_copy" not in s
-              and "move_tiles" not in s]
+              and "move_tiles" not in s and "move_pieces_hbm" not in s]   # kernel launch stubs, exported by the HIP compiler
     assert not leaked, leaked
 
 
