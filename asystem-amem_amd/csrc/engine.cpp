@@ -156,6 +156,7 @@ hipError_t Engine::reserve_pool(uint64_t bytes) {
   if (limit && bytes > limit) return hipErrorOutOfMemory;
   e = pool_->ensure(bytes);
   stats_.slab_bytes = pool_->capacity();
+  publish_stats();
   return e;
 }
 
@@ -782,6 +783,7 @@ hipError_t Engine::pause_copy_staged(Ctx& c, std::vector<Region*>& regs, bool* u
 
 int Engine::pause(Ctx& c, bool* rolled_back) {
   std::lock_guard<std::mutex> busy(busy_);
+  struct Publish { Engine* e; ~Publish() { e->publish_stats(); } } publish_on_return{this};
   auto t0 = Clock::now();
   if (rolled_back) *rolled_back = false;
   hipError_t e = init();
@@ -1043,6 +1045,7 @@ void Engine::forget(uint64_t va) {
 
 int Engine::resume(Ctx& c, bool* incomplete) {
   std::lock_guard<std::mutex> busy(busy_);
+  struct Publish { Engine* e; ~Publish() { e->publish_stats(); } } publish_on_return{this};
   if (incomplete) *incomplete = false;
   hipError_t e = init();
   if (e != hipSuccess) return (int)e;

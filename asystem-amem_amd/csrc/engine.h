@@ -82,7 +82,12 @@ class Engine {
   // A region was deleted while paused: drop its parked bytes.
   void forget(uint64_t va);
 
-  amem_cycle_stats stats() const { return stats_; }
+  // Figures of the last finished pause and resume. Another thread may ask while a cycle runs: it
+  // gets the snapshot published when the previous phase ended, never the record being filled in.
+  amem_cycle_stats stats() const {
+    std::lock_guard<std::mutex> lk(stats_mtx_);
+    return published_;
+  }
   uint64_t trim_pool();
   hipError_t reserve_pool(uint64_t bytes);
 
@@ -144,7 +149,13 @@ class Engine {
   bool ref_mode_ = false;    // the parked layout was made by the reference-structure path
   std::vector<uint8_t> parked_flags_;  // per-chunk zero flags of the last pause
 
-  amem_cycle_stats stats_ = {};
+  amem_cycle_stats stats_ = {};      // working record: written by the threads of the running cycle only
+  amem_cycle_stats published_ = {};  // what stats() hands out
+  mutable std::mutex stats_mtx_;
+  void publish_stats() {
+    std::lock_guard<std::mutex> lk(stats_mtx_);
+    published_ = stats_;
+  }
 };
 
 // Engine of a device, created on first use. Returns nullptr (after an ERROR log) when no

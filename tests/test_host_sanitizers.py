@@ -54,3 +54,32 @@ def test_registry_hammer_under_sanitizer(kind):
         assert "WARNING: ThreadSanitizer" not in r.stderr and "ERROR: AddressSanitizer" not in r.stderr, report
     finally:
         shutil.rmtree(outdir, ignore_errors=True)
+
+
+@pytest.mark.parametrize("kind", ["thread", "address"])
+def test_whole_cycles_with_imports_under_sanitizer(kind):
+    """The engine's own pause and resume under the sanitizers: the library's sources linked with the host
+    stand-in of the HIP calls (tests/host_standin), driven by tests/host_standin/cycle_driver.cpp through six
+    cycles with two importing ranks in the process, while three more threads hammer the hook and inspection
+    entry points. Every thread the engine starts (copy launcher, unmapper, releaser, three socket services)
+    is in the picture."""
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "tests", "host_standin"))
+    import build_standin
+    outdir = tempfile.mkdtemp(prefix="amem_san_cycle_")
+    try:
+        lib = build_standin.build(outdir, sanitize=kind)
+        exe = os.path.join(outdir, "cycle_driver_" + kind)
+        subprocess.run(["g++", "-O1", "-g", "-std=c++17", "-fsanitize=" + kind, "-fno-omit-frame-pointer",
+                        os.path.join(ROOT, "tests", "host_standin", "cycle_driver.cpp"), "-o", exe, lib,
+                        "-Wl,-rpath," + outdir, "-lpthread"], check=True, capture_output=True, text=True)
+        env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="1", GMM_IPC_DIR=outdir, AMEM_GROUPID=str(0x7800 + os.getpid() % 1000),
+                   TSAN_OPTIONS="exitcode=66 halt_on_error=0 report_signal_unsafe=0",
+                   ASAN_OPTIONS="exitcode=67 detect_leaks=0 protect_shadow_gap=0")
+        r = subprocess.run([exe], env=env, capture_output=True, text=True, timeout=600)
+        report = (r.stdout + r.stderr)[-8000:]
+        assert r.returncode == 0, report
+        assert "cycle driver done: 0 errors" in r.stdout, report
+        assert "WARNING: ThreadSanitizer" not in r.stderr and "ERROR: AddressSanitizer" not in r.stderr, report
+    finally:
+        shutil.rmtree(outdir, ignore_errors=True)
