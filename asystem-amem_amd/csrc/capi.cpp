@@ -334,6 +334,7 @@ int amem_update_peer_info(uint64_t va, int shared_fd) {
   if (!c) { if (shared_fd >= 0) close(shared_fd); return 1; }
   int dev = -1;
   size_t size = 0;
+  int state = AMEM_STATE_INVALID;
   {
     std::lock_guard<std::mutex> lf(c->fields);
     for (int d = 0; d < AMEM_MAX_DEVS && dev < 0; ++d) {
@@ -341,11 +342,21 @@ int amem_update_peer_info(uint64_t va, int shared_fd) {
       if (it == c->allocTable[d].end()) continue;
       dev = d;
       size = it->second.allocSz;
+      state = it->second.state;
     }
   }
   if (dev < 0) {
     LOGGER(ERROR, "groupID:%d pid:%d failed to find info for dptr:%llx to remap fd:%x", amem_groupID, getpid(),
            (unsigned long long)va, shared_fd);
+    if (shared_fd >= 0) close(shared_fd);
+    return 1;
+  }
+  // Only an address that a pause has emptied can take new memory. The CUDA driver refuses to map
+  // over an existing mapping; this HIP runtime accepts it (measured) and the old mapping would be
+  // lost without being unmapped, so the state is checked here.
+  if (state != AMEM_STATE_HOLE) {
+    LOGGER(ERROR, "groupID:%d pid:%d dptr:%llx is not released (state %d): refusing to map fd:%d over it", amem_groupID,
+           getpid(), (unsigned long long)va, state, shared_fd);
     if (shared_fd >= 0) close(shared_fd);
     return 1;
   }

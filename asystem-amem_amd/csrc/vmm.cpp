@@ -195,6 +195,15 @@ hipError_t vmm_export_fd(uint64_t handle, int* fd) {
 hipError_t vmm_import_map(int dev, uint64_t va, size_t size, int fd, bool close_fd,
                           uint64_t* new_handle) {
   hipMemGenericAllocationHandle_t h = nullptr;
+  // hipMemMap accepts an address that already holds a mapping (measured on ROCm 7.2) and the old
+  // mapping is then lost without having been unmapped: refuse here what the runtime does not.
+  if (vmm_is_mapped(va)) {
+    LOGGER(ERROR, "pid:%d curDev:%d dptr:%llx still holds a mapping; not importing inFD:%d over it", getpid(), dev,
+           (unsigned long long)va, fd);
+    if (close_fd) close(fd);
+    if (new_handle) *new_handle = 0;
+    return hipErrorInvalidValue;
+  }
   hipError_t e = CHECK_HIP(hipMemImportFromShareableHandle(&h, (void*)(uintptr_t)fd,
                                                            hipMemHandleTypePosixFileDescriptor));
   if (e == hipSuccess) {
