@@ -279,7 +279,10 @@ def main():
         "roofline": {"kernel": "scan_chunks (zero flags + checksums)", "bound": "hbm",
                      "achieved": round(k1_achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(k1_achieved / HBM_PEAK_GBPS, 4), "traffic": traffic, "traffic_from": traffic_from,
-                     "avg_launch_ms": round(k1_ms, 4), "algorithmic_bytes_per_launch": F},
+                     "avg_launch_ms": round(k1_ms, 4), "algorithmic_bytes_per_launch": F,
+                     "why_this_kernel": "the one kernel of a cycle that is bound by HBM; the two kernels that take over 99 % "
+                                        "of a cycle's GPU time move bytes over the host link, which is neither an HBM nor an MFMA "
+                                        "roofline: they are under link_kernels, against the measured link rate"},
         "link": {"measured_d2h_GBps": round(d2h.value, 2), "measured_h2d_GBps": round(h2d.value, 2),
                  "pause_leg_frac": round(pause_frac, 4),
                  "resume_leg_frac": round(resume_frac, 4),

@@ -176,3 +176,67 @@ def test_several_ranks_in_one_process_each_hold_a_slot():
         assert out["refused"] == 1
         assert out["table_size"] == 4 + 12 and out["peers_ok"]
         assert out["sockets_after"] == []
+
+
+def _service_under_garbage(ipc_dir, gid, to_parent, from_parent):
+    os.environ.update(AMEM_ENABLE="1", GMM_LOG="1", GMM_IPC_DIR=ipc_dir, AMEM_GROUPID=str(gid))
+    from asystem_amem_amd import binding as B, harness as H
+    lib = B.load()
+    assert lib.amem_add_alloc_info(OWNER_VA, 4 * MiB, B.TYPE_LOCAL, 0, OWNER_HANDLE, -1, 0, None, B.CALLER_P2P) == 0
+    to_parent.send(("slot", lib.amem_get_slot()))
+    assert from_parent.recv() == "check"
+    t = H.region_table(lib, 0)[OWNER_VA]
+    to_parent.send(("table", t["has_peer"], [p for p in t["peers"] if p], len(H.region_table(lib, 0))))
+    assert from_parent.recv() == "exit"
+    lib.amem_shutdown()
+
+
+def test_service_survives_malformed_and_abandoned_requests():
+    """Host-forced failures of the transport (the reference's worker asserts or spins on them,
+    gmm_worker_impl.cpp:288-431): a client that sends bytes that are no request, one that sends an unknown
+    operation, one that connects and goes away without a word. The service drops or answers each and keeps
+    serving: a well-formed registration afterwards still reaches the registry, and nothing else changed it."""
+    import socket
+    import struct
+    ctx = mp.get_context("spawn")
+    with tempfile.TemporaryDirectory() as ipc_dir:
+        gid = 0x7100 + os.getpid() % 2048
+        o_out, o_in = ctx.Pipe(), ctx.Pipe()
+        owner = ctx.Process(target=_service_under_garbage, args=(ipc_dir, gid, o_out[1], o_in[0]))
+        owner.start()
+        try:
+            assert o_out[0].poll(60)
+            tag, slot = o_out[0].recv()
+            path = os.path.join(ipc_dir, "amem_worker_%x_%d.sock" % (gid, slot))
+            # wire format of a request: magic "AMEM", op, sender slot, pid (4 x 32 bit), two 64-bit operands
+            def request(magic, op, sender, src, tgt):
+                return struct.pack("<IiiiQQ", magic, op, sender, os.getpid(), src, tgt)
+            MAGIC, REGISTER = 0x414D454D, 16
+            s1 = socket.socket(socket.AF_UNIX, socket.SOCK_STREAM); s1.connect(path)
+            s1.sendall(b"\x00" * 32)                                   # right length, wrong magic: dropped
+            s1.settimeout(5)
+            assert s1.recv(4) == b""                                   # the service closed the connection
+            s1.close()
+            s2 = socket.socket(socket.AF_UNIX, socket.SOCK_STREAM); s2.connect(path)
+            s2.close()                                                 # connected and left
+            s3 = socket.socket(socket.AF_UNIX, socket.SOCK_STREAM); s3.connect(path)
+            s3.settimeout(5)
+            s3.sendall(request(MAGIC, 99, 5, 0, 0))                    # unknown operation: answered with an error
+            assert struct.unpack("<i", s3.recv(4))[0] == 1
+            s3.sendall(request(MAGIC, REGISTER, 5, 0xDEAD, 0x7f5000000000))   # unknown handle: error, connection stays
+            assert struct.unpack("<i", s3.recv(4))[0] == 1
+            s3.sendall(request(MAGIC, REGISTER, 9, OWNER_HANDLE, 0x7f5000000000))   # slot out of range: error
+            assert struct.unpack("<i", s3.recv(4))[0] == 1
+            s3.sendall(request(MAGIC, REGISTER, 5, OWNER_HANDLE, 0x7f5000000000))   # and a good one on the same connection
+            assert struct.unpack("<i", s3.recv(4))[0] == 0
+            s3.close()
+            o_in[1].send("check")
+            assert o_out[0].poll(30)
+            tag, has_peer, peers, nregions = o_out[0].recv()
+            assert has_peer == 1 and peers == [0x7f5000000000] and nregions == 1
+            o_in[1].send("exit")
+            owner.join(30)
+            assert owner.exitcode == 0
+        finally:
+            if owner.is_alive():
+                owner.kill()
