@@ -10,7 +10,8 @@ two calls amem_mem_pause() and amem_mem_resume() and nothing else.
 Prints one JSON line:
   value      2 * F / (t_pause + t_resume), GB/s (1e9), F = registered footprint bytes
   pause_leg_frac_of_link / resume_leg_frac_of_link   bytes that crossed the host link in the leg over
-             (leg time x measured hipMemcpy rate): the figures the 80 % target is about
+             (leg time x measured hipMemcpy rate): the figures the 80 % target is about;
+             both_legs_frac_of_link is the same for the whole cycle (bytes of both legs over both times)
   roofline   the on-device scan kernel (zero flags + checksums) against HBM peak
   link       each leg against the measured hipMemcpy rate of the host link
   link_kernels  the two kernels that take nearly all GPU time, gather-pack and scatter-unpack against pinned
@@ -250,6 +251,7 @@ def main():
         "unit": "GB/s",
         "pause_leg_frac_of_link": round(pause_frac, 4),
         "resume_leg_frac_of_link": round(resume_frac, 4),
+        "both_legs_frac_of_link": round(2 * parked / (p50_pause + p50_resume) / 1e9 / ((d2h.value + h2d.value) / 2), 4),
         "leg_frac_target": 0.8,
         "legs_meeting_target": [n for n, f in (("pause", pause_frac), ("resume", resume_frac)) if f >= 0.8],
         "n_gpus": 1,
