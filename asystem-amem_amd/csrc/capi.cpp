@@ -626,6 +626,7 @@ static OptRef* opt_table(size_t* n) {
       {"hbm_wgs", &o.hbm_wgs, 1, 1 << 20},
       {"hbm_move_wgs", &o.hbm_move_wgs, 1, (int64_t)1 << 30},
       {"resume_batch_bytes", &o.resume_batch_bytes, 1, (int64_t)1 << 40},
+      {"resume_dma_min_bytes", &o.resume_dma_min_bytes, 0, (int64_t)1 << 40},
       {"peer_timeout_ms", &o.peer_timeout_ms, 0, (int64_t)1 << 40},
       {"peer_loopback", &o.peer_loopback, 0, 1},
       {"offload_free_tag", &o.offload_free_tag, -1, AMEM_MAX_CALLER - 1},

@@ -1077,9 +1077,13 @@ int Engine::resume(Ctx& c, bool* incomplete) {
   }
 
   // Scatter list: per region, its parked runs and its zero runs.
-  struct Item { Region* r; uint64_t va; uint32_t d0, d1; uint64_t bytes; };
+  struct Item { Region* r; uint64_t va; uint32_t d0, d1; uint64_t bytes; uint32_t m0, m1; };
   std::vector<Item> items;
   std::vector<CopyDesc> scatter;
+  // Runs at least resume_dma_min_bytes long (0 = none) come back by hipMemcpyAsync on the second
+  // stream, next to the scatter kernel on the first; `dma` holds them, an item's are [m0, m1).
+  std::vector<CopyDesc> dma;
+  const uint64_t dma_min = ref_mode_ ? 0 : (uint64_t)options().resume_dma_min_bytes;
   const uint8_t* flags = parked_flags_.data();
   const uint64_t slab_bytes = pool_->slab_bytes();
   std::vector<ScanSeg> verify_segs;
@@ -1090,12 +1094,21 @@ int Engine::resume(Ctx& c, bool* incomplete) {
     if (it == table.end()) continue;
     Region& r = it->second;
     if (r.state != AMEM_STATE_HOLE || from_peer(r.type)) continue;
-    Item im = {&r, p.va, (uint32_t)scatter.size(), 0, p.size};
+    Item im = {&r, p.va, (uint32_t)scatter.size(), 0, p.size, (uint32_t)dma.size(), 0};
     uint64_t cursor = p.parked_off;
     std::vector<CopyDesc> zeros;
     emit_runs(flags + p.first_chunk, p.va, p.size, elide || p.skip, &cursor, slab_bytes, &scatter, &zeros, nullptr);
+    if (dma_min) {
+      size_t keep = im.d0;
+      for (size_t d = im.d0; d < scatter.size(); ++d) {
+        if (scatter[d].bytes >= dma_min) dma.push_back(scatter[d]);
+        else scatter[keep++] = scatter[d];
+      }
+      scatter.resize(keep);
+    }
     scatter.insert(scatter.end(), zeros.begin(), zeros.end());
     im.d1 = (uint32_t)scatter.size();
+    im.m1 = (uint32_t)dma.size();
     items.push_back(im);
     if (p.skip) continue;  // scratch regions come back as zeros by design: nothing to compare against
     verify_segs.push_back({p.va, p.size});
@@ -1108,7 +1121,7 @@ int Engine::resume(Ctx& c, bool* incomplete) {
     Region& r = kv.second;
     if (r.state != AMEM_STATE_HOLE || from_peer(r.type)) continue;
     if (item_vas.count(kv.first)) continue;
-    Item im = {&r, kv.first, (uint32_t)scatter.size(), 0, (uint64_t)r.allocSz};
+    Item im = {&r, kv.first, (uint32_t)scatter.size(), 0, (uint64_t)r.allocSz, (uint32_t)dma.size(), (uint32_t)dma.size()};
     scatter.push_back({kv.first, kDescZero, (uint64_t)r.allocSz & ~(uint64_t)15});
     im.d1 = (uint32_t)scatter.size();
     items.push_back(im);
@@ -1166,6 +1179,11 @@ int Engine::resume(Ctx& c, bool* incomplete) {
         }
         note(CHECK_HIP(hipStreamSynchronize(dstream_)));
       }
+      for (uint32_t m = im.m0; m < im.m1 && rc == 0; ++m) {
+        note(CHECK_HIP(hipMemcpyAsync((void*)(uintptr_t)dma[m].va, pool_->host_addr(dma[m].off), dma[m].bytes,
+                                      hipMemcpyHostToDevice, dstream_)));
+        stats_.dma_bytes += dma[m].bytes;
+      }
       bytes += im.bytes;
       ++j;
     }
@@ -1189,6 +1207,7 @@ int Engine::resume(Ctx& c, bool* incomplete) {
     i = j;
   }
   note(CHECK_HIP(hipStreamSynchronize(kstream_)));
+  if (!dma.empty()) note(CHECK_HIP(hipStreamSynchronize(dstream_)));
   stats_.resume_copy_ms = ms_since(tc);
   for (auto& pr : timed) {
     float ms = 0;

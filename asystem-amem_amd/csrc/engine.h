@@ -32,6 +32,7 @@ struct Options {
   int64_t hbm_wgs = 65536;                // workgroup cap of the scan kernel
   int64_t hbm_move_wgs = 1 << 22;         // workgroup cap of the mover when both sides are device memory
   int64_t resume_batch_bytes = 64ll << 20;
+  int64_t resume_dma_min_bytes = 0;       // resume: runs this long come back by hipMemcpyAsync on the second stream (0 = none)
   int64_t peer_timeout_ms = 60000;
   int64_t release_thread = 1;             // interleaved path: handles are released on a third thread
   int64_t scratch_on_host = 0;            // 1: engine tables live in pinned host memory even if the device has room

@@ -296,6 +296,10 @@ int amem_set_enabled(int on);
  *                     (default 4194304: one workgroup per 4 KiB piece up to 16 GiB, striding beyond)
  *   "resume_batch_bytes" resume maps regions in batches of about this many bytes and follows each
  *                     batch with one unpack launch (default 64 MiB)
+ *   "resume_dma_min_bytes" resume brings runs of parked bytes at least this long back with
+ *                     hipMemcpyAsync on a second stream while the unpack kernel handles the shorter ones
+ *                     and the zero fill on the first (default 0: everything goes through the kernel,
+ *                     which measured 2 % below the copy engine's rate and needs no second stream)
  *   "peer_timeout_ms" how long resume waits for owners before failing (0 = forever)
  *   "offload_free_tag" caller tag (0-15, -1 = none) whose regions hold scratch data: pause releases
  *                     them without copying and resume hands them back zero-filled. This is what

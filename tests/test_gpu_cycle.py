@@ -21,7 +21,7 @@ GiB = 1 << 30
 def eng(gpu, fresh):
     defaults = {k: fresh.amem_get_option(k) for k in (b"zero_elide", b"verify", b"pause_path", b"dma_min_bytes",
                                                        b"staging_bytes", b"resume_batch_bytes", b"scratch_on_host", b"release_thread",
-                                                       b"pause_wgs", b"pause_xcds", b"interleave_bytes")}
+                                                       b"pause_wgs", b"pause_xcds", b"interleave_bytes", b"resume_dma_min_bytes")}
     yield fresh
     fresh.amem_mem_resume(0, 0)        # a test that failed mid-cycle must not leave the engine paused
     for k, v in defaults.items():
@@ -127,7 +127,9 @@ def test_repeated_cycles_with_writes_between(eng):
                                   {"staging_bytes": 8 << 20}, {"resume_batch_bytes": 1},
                                   {"staging_bytes": 1 << 20, "resume_batch_bytes": 1 << 40},
                                   {"pause_path": 3, "interleave_bytes": 1 << 16}, {"pause_path": 4},
-                                  {"release_thread": 0}, {"release_thread": 0, "pause_wgs": 96, "pause_xcds": 8}])
+                                  {"release_thread": 0}, {"release_thread": 0, "pause_wgs": 96, "pause_xcds": 8},
+                                  {"resume_dma_min_bytes": 128 << 10}, {"resume_dma_min_bytes": 1 << 16, "pause_path": 0, "dma_min_bytes": 128 << 10},
+                                  {"resume_dma_min_bytes": 1 << 16, "zero_elide": 0}])
 def test_option_paths_are_all_bit_exact(eng, opts):
     lib = eng
     for k, v in opts.items():
@@ -147,6 +149,10 @@ def test_option_paths_are_all_bit_exact(eng, opts):
         if opts.get("staging_bytes") == 1 << 20:
             assert st["kernel_bytes"] > 0                   # regions larger than a staging buffer go direct
         assert lib.amem_mem_resume(0, 0) == 0
+        if opts.get("resume_dma_min_bytes"):                  # some runs came back by the copy engine, the rest by the kernel
+            back = H.cycle_stats(lib)["dma_bytes"] - st["dma_bytes"]
+            assert 0 < back <= st["parked_bytes"]
+            assert H.cycle_stats(lib)["k3_launches"] > 0 or opts.get("zero_elide") == 0   # (no zero runs to fill: nothing left for the kernel)
         assert regs.mismatched_bytes() == 0
     after = regs.table()
     assert [d for d in H.compare_tables(before, after) if d[1] != "handle_gen"] == []
