@@ -27,6 +27,17 @@
 // and the dma-buf export of the HSA runtime through dlopen + dlsym on explicit handles, which no
 // library placed in front of them can intercept; a patched RCCL calls amem_delAllocInfo there itself.
 //
+//   hipMalloc / hipFree            only with AMEM_HOOK_PLAIN_ALLOC=<bytes> in the environment (off by default):
+//                                  an RCCL build that keeps its buffers in plain allocations (the one ROCm 7.2
+//                                  ships does, whatever NCCL_CUMEM_ENABLE says) gives the engine nothing it
+//                                  could release. With the variable set, hipMalloc calls of at least that many
+//                                  bytes coming from RCCL are served through the virtual-memory API instead
+//                                  (reserve, create, map, grant access: what ncclCuMemAlloc would have done)
+//                                  and registered, and hipFree of such an address undoes it. Memory served
+//                                  this way cannot be shared through hipIpcGetMemHandle, so the switch is
+//                                  for layouts in which RCCL does not hand these buffers to another process
+//                                  over legacy IPC (one rank per node, or P2P over IPC disabled).
+//
 // Calls made by anything else (the pause/resume engine itself, the application) pass through
 // untouched. The module a call comes from is found from its return address.
 #define _GNU_SOURCE 1
@@ -288,6 +299,89 @@ HOOK_API hipError_t hipMemRelease(hipMemGenericAllocationHandle_t handle) {
     if (!id.empty()) unlink(export_file(id).c_str());
   }
   return fn(handle);
+}
+
+// ---- plain allocations served through the virtual-memory API (opt-in) ----
+
+namespace {
+std::unordered_map<uint64_t, uint64_t> g_substituted;  // address handed to RCCL -> mapped size
+long long g_plain_min = -2;
+size_t plain_alloc_min() {
+  if (g_plain_min == -2) {
+    const char* e = getenv("AMEM_HOOK_PLAIN_ALLOC");
+    g_plain_min = (e && atoll(e) > 0) ? atoll(e) : 0;
+  }
+  return (size_t)g_plain_min;
+}
+}  // namespace
+
+// Serve one plain allocation of RCCL's through the virtual-memory API and register it. False when that
+// is not possible, in which case the caller falls back to the ordinary allocation.
+static bool serve_plain(void** ptr, size_t size) {
+  int dev = 0;
+  (void)hipGetDevice(&dev);
+  uint64_t va = 0, handle = 0, asz = 0;
+  if (amem_vmm_alloc(size, dev, &va, &handle, &asz) != 0) return false;  // no room that way: the plain way decides
+  // the shape of the reference's hook in ncclCuMemAlloc (nccl_patch/nccl_2.27.5-1.diff:278-280)
+  const int rc = amem_add_alloc_info(va, asz, AMEM_TYPE_LOCAL, dev, handle, -1, 0, NULL, AMEM_CALLER_DEFAULT);
+  {
+    std::lock_guard<std::mutex> lk(g_mtx);
+    g_substituted[va] = asz;
+    if (rc == 0) g_registered.insert(va);
+  }
+  if (verbose()) fprintf(stderr, "AMEM [DEBG] rccl_hook: plain allocation of %zu bytes served as a mapping at %llx of %llu bytes, registered rc %d\n",
+                         size, (unsigned long long)va, (unsigned long long)asz, rc);
+  *ptr = (void*)(uintptr_t)va;
+  return true;
+}
+
+HOOK_API hipError_t hipMalloc(void** ptr, size_t size) {
+  static auto fn = real<hipError_t (*)(void**, size_t)>("hipMalloc");
+  const size_t min = plain_alloc_min();
+  if (min && ptr && size >= min && from_rccl(__builtin_return_address(0)) && serve_plain(ptr, size)) return hipSuccess;
+  return fn(ptr, size);
+}
+
+HOOK_API hipError_t hipFree(void* ptr) {
+  static auto fn = real<hipError_t (*)(void*)>("hipFree");
+  uint64_t asz = 0;
+  bool was_registered = false;
+  if (ptr) {
+    std::lock_guard<std::mutex> lk(g_mtx);
+    auto it = g_substituted.find((uint64_t)(uintptr_t)ptr);
+    if (it != g_substituted.end()) {
+      asz = it->second;
+      g_substituted.erase(it);
+      was_registered = g_registered.erase((uint64_t)(uintptr_t)ptr) > 0;
+    }
+  }
+  if (!asz) return fn(ptr);
+  (void)hipDeviceSynchronize();  // hipFree waits for the device; so does this
+  if (was_registered) (void)amem_del_alloc_info((uint64_t)(uintptr_t)ptr, 0, 0);
+  const int rc = amem_vmm_free((uint64_t)(uintptr_t)ptr, asz, 0);  // works for a paused (unmapped) address too
+  if (verbose()) fprintf(stderr, "AMEM [DEBG] rccl_hook: hipFree(%p) of a served mapping, %llu bytes, rc %d\n", ptr,
+                         (unsigned long long)asz, rc);
+  return rc == 0 ? hipSuccess : hipErrorInvalidValue;
+}
+
+HOOK_API hipError_t hipExtMallocWithFlags(void** ptr, size_t size, unsigned int flags) {
+  static auto fn = real<hipError_t (*)(void**, size_t, unsigned int)>("hipExtMallocWithFlags");
+  // flags 0 is an ordinary allocation under another name (this is how RCCL 2.27 allocates everything);
+  // fine-grained, uncached and signal memory keep their own semantics and are never served differently
+  const size_t min = plain_alloc_min();
+  const bool rccl = (min || verbose()) && from_rccl(__builtin_return_address(0));
+  if (rccl && min && ptr && flags == hipDeviceMallocDefault && size >= min && serve_plain(ptr, size)) return hipSuccess;
+  if (rccl && verbose() && size >= (1u << 20))
+    fprintf(stderr, "AMEM [DEBG] rccl_hook: hipExtMallocWithFlags(%zu, flags %x) left as it is\n", size, flags);
+  return fn(ptr, size, flags);
+}
+
+// Bytes currently served to RCCL through the virtual-memory API in place of plain allocations.
+HOOK_API uint64_t amem_rccl_hook_served_bytes(void) {
+  std::lock_guard<std::mutex> lk(g_mtx);
+  uint64_t n = 0;
+  for (auto& kv : g_substituted) n += kv.second;
+  return n;
 }
 
 // Number of RCCL mappings currently mirrored into the registry (for tests and diagnostics).

@@ -259,7 +259,8 @@ def test_rccl_hook_library_exports_the_interposed_calls():
     out = subprocess.run(["nm", "-D", "--defined-only", hook], check=True, capture_output=True, text=True).stdout
     names = {l.split()[-1] for l in out.splitlines() if " T " in l}
     assert names == {"hipMemMap", "hipMemSetAccess", "hipMemUnmap", "hipMemImportFromShareableHandle",
-                     "hipMemExportToShareableHandle", "hipMemRelease", "amem_rccl_hook_registered"}
+                     "hipMemExportToShareableHandle", "hipMemRelease", "hipMalloc", "hipFree", "hipExtMallocWithFlags",
+                     "amem_rccl_hook_registered", "amem_rccl_hook_served_bytes"}
     # unversioned definitions: they satisfy librccl's versioned references (hipMemMap@hip_5.1 ...)
     assert "@" not in "".join(names)
 

@@ -254,3 +254,89 @@ def test_hook_registers_imported_mappings_with_their_owner(gpu, tmp_path):
     env.pop("AMEM_IPC", None)
     r = subprocess.run([sys.executable, "-c", IMPORT_CHILD, ROOT, standin], env=env, capture_output=True, text=True, timeout=240)
     assert r.returncode == 0 and "rccl hook import side ok" in r.stdout, (r.returncode, r.stdout[-3000:], r.stderr[-3000:])
+
+
+PLAIN_ALLOC_CHILD = r'''
+import ctypes as C, os, sys
+import numpy as np
+root = sys.argv[1]
+sys.path.insert(0, root)
+libdir = os.path.join(root, "asystem-amem_amd", "lib")
+hook = C.CDLL(os.path.join(libdir, "libamem_rccl_hook.so"), mode=C.RTLD_GLOBAL)   # before the runtime and RCCL
+from asystem_amem_amd import binding as B, harness as H
+lib = B.load()
+hip = C.CDLL("libamdhip64.so")
+try:
+    rccl = C.CDLL("librccl.so")
+except OSError as e:
+    print("no librccl.so:", e); print("rccl skipped"); sys.exit(0)
+hook.amem_rccl_hook_registered.restype = C.c_int64
+hook.amem_rccl_hook_served_bytes.restype = C.c_uint64
+class UID(C.Structure):
+    _fields_ = [("b", C.c_char * 128)]
+rccl.ncclCommInitRank.argtypes = [C.POINTER(C.c_void_p), C.c_int, UID, C.c_int]
+rccl.ncclAllReduce.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+rccl.ncclCommDestroy.argtypes = [C.c_void_p]
+assert hip.hipSetDevice(0) == 0
+uid, comm = UID(), C.c_void_p()
+assert rccl.ncclGetUniqueId(C.byref(uid)) == 0
+assert rccl.ncclCommInitRank(C.byref(comm), 1, uid, 0) == 0
+served, regions = hook.amem_rccl_hook_served_bytes(), hook.amem_rccl_hook_registered()
+print("served to RCCL through the virtual-memory API: %.1f MiB in %d regions" % (served / 2**20, regions))
+if served == 0:
+    print("this RCCL made no plain allocation of 1 MiB or more"); print("rccl skipped"); sys.exit(0)
+assert lib.amem_region_count(0) == regions
+tab = H.region_table(lib, 0)
+assert sum(t["alloc_sz"] for t in tab.values()) == served and all(t["type"] == B.TYPE_LOCAL for t in tab.values())
+MiB = 1 << 20
+n = 4 * MiB // 4
+bufs = []
+for _ in range(2):
+    p = C.c_void_p()
+    assert hip.hipMalloc(C.byref(p), 4 * MiB) == 0     # the application's own buffers: ordinary memory, not the hook's business
+    bufs.append(p.value)
+send, recv = bufs
+assert lib.amem_region_count(0) == regions
+rng = np.random.default_rng(6)
+
+def allreduce_wrong():
+    x = rng.standard_normal(n).astype(np.float32)
+    assert lib.amem_copy_to_device(send, x.ctypes.data, x.nbytes) == 0
+    junk = np.full(n, -1.0, dtype=np.float32)
+    assert lib.amem_copy_to_device(recv, junk.ctypes.data, junk.nbytes) == 0
+    assert rccl.ncclAllReduce(send, recv, n, 7, 0, comm, None) == 0            # ncclFloat32, ncclSum, null stream
+    assert hip.hipDeviceSynchronize() == 0
+    y = np.empty_like(x)
+    assert lib.amem_copy_from_device(y.ctypes.data, recv, y.nbytes) == 0
+    return int(np.count_nonzero(x != y))
+
+assert allreduce_wrong() == 0
+lib.ncclPause(None); lib.ncclResume(None)                                      # warm cycle
+for cycle in range(3):
+    free0 = H.mem_free(lib)
+    assert lib.ncclPause(None) == 0 and lib.amem_check_paused(0) == 1
+    released = H.mem_free(lib) - free0
+    assert released >= served - 2 * MiB, (released, served)                    # the communicator's own memory is gone
+    assert lib.ncclResume(None) == 0 and lib.amem_check_paused(0) == 0
+    assert allreduce_wrong() == 0, cycle                                       # the same communicator still works
+assert rccl.ncclCommDestroy(comm) == 0                                         # RCCL frees what it was served
+assert hook.amem_rccl_hook_served_bytes() == 0 and hook.amem_rccl_hook_registered() == 0 and lib.amem_region_count(0) == 0
+print("released per pause: %.1f MiB" % (released / 2**20))
+print("rccl plain ok")
+'''
+
+
+def test_real_rccl_buffers_served_through_the_vmm_api_are_released_and_restored(gpu):
+    """A real communicator's own memory in the registry (what the reference's hooks in ncclCuMemAlloc are
+    for, nccl_patch/nccl_2.27.5-1.diff:278-280). The RCCL of this ROCm release keeps its buffers in plain
+    allocations, which nothing can unmap; with AMEM_HOOK_PLAIN_ALLOC set, the hook serves RCCL's plain
+    allocations of at least that size through the virtual-memory API and registers them. A one-rank
+    communicator then really gives its memory back at ncclPause, gets it back at ncclResume at the same
+    addresses, and an all-reduce through it is right after each of three cycles (the check of
+    nccl_patch/nccl-tests.diff:24-50). Uncached and fine-grained allocations are left alone."""
+    env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="1", AMEM_IPC="0", AMEM_HOOK_PLAIN_ALLOC=str(1 << 20))
+    r = subprocess.run([sys.executable, "-c", PLAIN_ALLOC_CHILD, ROOT], env=env, capture_output=True, text=True, timeout=240)
+    assert r.returncode == 0 and ("rccl plain ok" in r.stdout or "rccl skipped" in r.stdout), \
+        (r.returncode, r.stdout[-3000:], r.stderr[-3000:])
+    if "rccl skipped" in r.stdout:
+        pytest.skip("librccl.so is not loadable here, or it made no plain allocation the hook serves")
