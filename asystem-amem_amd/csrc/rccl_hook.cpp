@@ -42,6 +42,7 @@
 // untouched. The module a call comes from is found from its return address.
 #define _GNU_SOURCE 1
 #include <dlfcn.h>
+#include <fcntl.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -228,19 +229,27 @@ HOOK_API hipError_t hipMemImportFromShareableHandle(hipMemGenericAllocationHandl
     if (shHandleType == hipMemHandleTypePosixFileDescriptor) {
       const std::string id = identity_of((int)(uintptr_t)osHandle);
       bool found = false;
-      if (!id.empty()) {
+      // (AMEM_HOOK_NOTES_ONLY makes an importer look at the notes even for descriptors its own process
+      // exported, the way an importer in another process has to: for tests of that path)
+      static const bool notes_only = getenv("AMEM_HOOK_NOTES_ONLY") != nullptr;
+      if (!id.empty() && !notes_only) {
         std::lock_guard<std::mutex> lk(g_mtx);
         auto it = g_exports.find(id);
         if (it != g_exports.end()) { owner = it->second; found = true; }
       }
       if (!found && !id.empty()) {
         // exported by another process: it left a note under the descriptor's identity
-        if (FILE* f = fopen(export_file(id).c_str(), "r")) {
+        // (only a note this user wrote counts, and a symbolic link in its place is not followed)
+        const int nfd = open(export_file(id).c_str(), O_RDONLY | O_NOFOLLOW | O_CLOEXEC);
+        struct stat st;
+        if (nfd >= 0 && fstat(nfd, &st) == 0 && S_ISREG(st.st_mode) && st.st_uid == geteuid()) {
+          char buf[96] = {0};
+          const ssize_t n = read(nfd, buf, sizeof(buf) - 1);
           int slot = -1;
           unsigned long long h = 0;
-          if (fscanf(f, "%d %llx", &slot, &h) == 2) owner = {slot, (uint64_t)h};
-          fclose(f);
+          if (n > 0 && sscanf(buf, "%d %llx", &slot, &h) == 2 && slot >= 0 && slot < AMEM_MAX_DEVS) owner = {slot, (uint64_t)h};
         }
+        if (nfd >= 0) close(nfd);
       }
     }
     if (verbose()) fprintf(stderr, "AMEM [DEBG] rccl_hook: imported handle %p, owner slot %d handle %llx\n", (void*)*handle,
@@ -274,9 +283,15 @@ HOOK_API hipError_t hipMemExportToShareableHandle(void* shareableHandle, hipMemG
         if (uint64_t va = amem_handle_lookup(dev, h)) g_export_at[va] = id;
       }
       if (!stale.empty()) unlink(export_file(stale).c_str());
-      if (FILE* f = fopen(export_file(id).c_str(), "w")) {
-        fprintf(f, "%d %llx %d\n", slot, (unsigned long long)h, (int)getpid());
-        fclose(f);
+      // the note is this user's alone, and is never written through a link somebody else left under its name
+      const std::string note = export_file(id);
+      unlink(note.c_str());
+      const int nfd = open(note.c_str(), O_WRONLY | O_CREAT | O_EXCL | O_NOFOLLOW | O_CLOEXEC, 0600);
+      if (nfd >= 0) {
+        char buf[96];
+        const int n = snprintf(buf, sizeof(buf), "%d %llx %d\n", slot, (unsigned long long)h, (int)getpid());
+        if (write(nfd, buf, (size_t)n) != n && verbose()) fprintf(stderr, "AMEM [WARN] rccl_hook: short write to %s\n", note.c_str());
+        close(nfd);
       }
       if (verbose()) fprintf(stderr, "AMEM [DEBG] rccl_hook: exported handle %p as %s (slot %d)\n", (void*)handle, id.c_str(), slot);
     }

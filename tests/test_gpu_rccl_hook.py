@@ -239,12 +239,15 @@ print("rccl hook import side ok")
 '''
 
 
-def test_hook_registers_imported_mappings_with_their_owner(gpu, tmp_path):
+@pytest.mark.parametrize("via", ["memory", "notes"])
+def test_hook_registers_imported_mappings_with_their_owner(gpu, tmp_path, via):
     """The importer's half of the hook (the reference's site in ncclP2pImportShareableBuffer,
     nccl_patch/nccl_2.27.5-1.diff:572-579): a second rank, living in the same process under a slot of its
     own, imports the descriptors the first rank exports; the hook names the owner from the descriptor's
     identity and registers each mapping as PEER_POSIX, so a pause drops the importer's mappings before
-    the owner's release and a resume maps the new memory back at the importer's addresses."""
+    the owner's release and a resume maps the new memory back at the importer's addresses.
+    "notes": the importer finds the owner through the note files under GMM_IPC_DIR, as an importer in
+    another process has to, instead of through what its own process remembers of its exports."""
     standin = str(tmp_path / "librccl_standin.so")
     rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
     subprocess.run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-D__HIP_PLATFORM_AMD__",
@@ -252,6 +255,8 @@ def test_hook_registers_imported_mappings_with_their_owner(gpu, tmp_path):
                     "-o", standin, "-L" + os.path.join(rocm, "lib"), "-lamdhip64"], check=True, capture_output=True, text=True)
     env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="1", GMM_IPC_DIR=str(tmp_path), AMEM_GROUPID=str(0x7400 + os.getpid() % 1024))
     env.pop("AMEM_IPC", None)
+    if via == "notes":
+        env["AMEM_HOOK_NOTES_ONLY"] = "1"
     r = subprocess.run([sys.executable, "-c", IMPORT_CHILD, ROOT, standin], env=env, capture_output=True, text=True, timeout=240)
     assert r.returncode == 0 and "rccl hook import side ok" in r.stdout, (r.returncode, r.stdout[-3000:], r.stderr[-3000:])
 
