@@ -225,7 +225,7 @@ bool claim(int slot, Service& g_svc) {
   for (int attempt = 0; attempt < 4; ++attempt) {
     // Only this user's processes form a group (the service refuses everybody else), so nobody
     // else needs to open the lock, and nobody else should be able to hold it and fake a live peer.
-    int fd = open(lp.c_str(), O_CREAT | O_RDWR | O_CLOEXEC, 0600);
+    int fd = open(lp.c_str(), O_CREAT | O_RDWR | O_CLOEXEC | O_NOFOLLOW, 0600);
     if (fd < 0) return false;
     if (flock(fd, LOCK_EX | LOCK_NB) != 0) { close(fd); return false; }
     // The lock is on the file, not on its name: if the name was removed or replaced between the
@@ -245,7 +245,7 @@ bool claim(int slot, Service& g_svc) {
 // True while some process holds the lock file of `slot`. The lock dies with its holder, so
 // this is how a peer that crashed is told from one that is merely slow.
 bool slot_claimed(int slot) {
-  int fd = open(lock_name(slot).c_str(), O_RDWR | O_CLOEXEC);
+  int fd = open(lock_name(slot).c_str(), O_RDWR | O_CLOEXEC | O_NOFOLLOW);
   if (fd < 0) return false;
   const bool held = flock(fd, LOCK_SH | LOCK_NB) != 0;
   if (!held) flock(fd, LOCK_UN);
