@@ -268,6 +268,7 @@ def main():
         "p50_pause_s": round(p50_pause, 4),
         "p50_resume_s": round(p50_resume, 4),
         "p50_cycle_s": round(statistics.median(a + b for a, b in zip(pause_s, resume_s)), 4),
+        "max_pause_s": round(max(pause_s), 4), "max_resume_s": round(max(resume_s), 4),
         "first_cycle_s": {"pause": round(first[0], 4), "resume": round(first[1], 4)} if args.warmup else None,
         "first_cycle": {"pause_s": round(first[0], 4), "resume_s": round(first[1], 4),
                         "phases_ms": {k: round(first[2][k], 3) for k in PHASES},
