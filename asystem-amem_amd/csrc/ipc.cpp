@@ -75,8 +75,8 @@ Service& g_svc = g_ipc.primary;
 // The slot on whose behalf this thread registers imported regions; -1 = the primary slot.
 thread_local int t_acting_slot = -1;
 
-// Whether `slot` is one of this process's own (callers need not hold g_ipc.mtx: slots are only
-// added while no peer traffic of theirs exists, and read as plain ints).
+// Whether `slot` is one of this process's own. Takes g_ipc.mtx for the extra slots: callers must
+// not hold it (none of the service threads' handlers comes here, so ipc_stop may join them under it).
 bool own_slot(int slot) {
   if (slot < 0) return false;
   if (g_svc.slot == slot) return true;
