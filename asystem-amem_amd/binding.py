@@ -148,7 +148,7 @@ def load(path=None):
     global _lib
     if _lib is not None:
         return _lib
-    path = path or os.environ.get("AMEM_LIB", LIB_PATH)
+    path = path or LIB_PATH   # no environment override: the package only ever loads the library it ships
     if not os.path.exists(path):
         raise RuntimeError(
             "%s is missing: build it with `python asystem-amem_amd/build.py` "

@@ -113,7 +113,7 @@ def main():
     H.enable_env()
     import __graft_entry__
     __graft_entry__.ensure_built()      # loads what is built; compiles only if a library is missing
-    lib = B.load(B.LIB_PATH)            # the shipped library, whatever AMEM_LIB says
+    lib = B.load()
     if lib.amem_device_count() < 1:
         sys.exit("bench.py needs a GPU")
     if args.pause_path is not None:

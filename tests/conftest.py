@@ -33,8 +33,10 @@ def _libraries():
 
 @pytest.fixture(scope="session")
 def lib():
+    """The shipped library. Only the child pytest of tests/test_engine_on_host_standin.py sets
+    AMEM_TEST_LIB, to run engine-logic tests against the test-only build on the host stand-in."""
     from asystem_amem_amd import binding
-    return binding.load()
+    return binding.load(os.environ.get("AMEM_TEST_LIB") or None)
 
 
 @pytest.fixture(scope="session")

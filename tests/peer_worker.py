@@ -26,11 +26,9 @@ def _worker(rank, world, ipc_dir, gid, conns, ctrl, lib_path=None):
     lib_path: library to load instead of the shipped one (the host stand-in build)."""
     try:
         os.environ.update(AMEM_ENABLE="1", GMM_LOG="2", GMM_IPC_DIR=ipc_dir, AMEM_GROUPID=str(gid), AMEM_SLOT=str(rank))
-        if lib_path:
-            os.environ["AMEM_LIB"] = lib_path
         from asystem_amem_amd import binding as B, harness as H
         from asystem_amem_amd.footprint import Footprint
-        lib = B.load()
+        lib = B.load(lib_path)
         lib.amem_set_option(b"peer_timeout_ms", 60000)
         fp = Footprint(2, 4 + rank, max_regions=NREG, threads=2)
         regs = H.Regions(lib, fp)                      # local regions, registered

@@ -21,7 +21,7 @@ SELECTION = ("option_paths or state_machine_edges or rolls_back or stale_registr
 def test_engine_logic_tests_pass_on_the_host_standin():
     import build_standin
     lib = build_standin.build(os.path.join(HERE, "host_standin", "_build"))
-    env = dict(os.environ, AMEM_LIB=lib, AMEM_ENABLE="1", GMM_LOG="1")
+    env = dict(os.environ, AMEM_TEST_LIB=lib, AMEM_ENABLE="1", GMM_LOG="1")
     r = subprocess.run([sys.executable, "-m", "pytest", "-q", "-x", "-m", "gpu", "-p", "no:cacheprovider", "-k", SELECTION,
                         os.path.join(HERE, "test_gpu_cycle.py"), os.path.join(HERE, "test_gpu_kernels.py"),
                         os.path.join(HERE, "test_zz_no_alloc.py")],

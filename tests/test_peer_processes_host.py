@@ -39,10 +39,10 @@ def test_processes_through_pause_and_resume(standin, world):
 
 
 def _owner_that_dies(ipc_dir, gid, lib_path, conn, ctrl):
-    os.environ.update(AMEM_ENABLE="1", GMM_LOG="1", GMM_IPC_DIR=ipc_dir, AMEM_GROUPID=str(gid), AMEM_SLOT="0", AMEM_LIB=lib_path)
+    os.environ.update(AMEM_ENABLE="1", GMM_LOG="1", GMM_IPC_DIR=ipc_dir, AMEM_GROUPID=str(gid), AMEM_SLOT="0")
     from asystem_amem_amd import binding as B, harness as H
     from asystem_amem_amd.footprint import Footprint
-    lib = B.load()
+    lib = B.load(lib_path)
     fp = Footprint(2, 31, max_regions=3, threads=2)
     regs = H.Regions(lib, fp)
     for i in range(3):
@@ -59,10 +59,10 @@ def _owner_that_dies(ipc_dir, gid, lib_path, conn, ctrl):
 
 
 def _importer_of_a_dead_owner(ipc_dir, gid, lib_path, conn, ctrl):
-    os.environ.update(AMEM_ENABLE="1", GMM_LOG="1", GMM_IPC_DIR=ipc_dir, AMEM_GROUPID=str(gid), AMEM_SLOT="1", AMEM_LIB=lib_path)
+    os.environ.update(AMEM_ENABLE="1", GMM_LOG="1", GMM_IPC_DIR=ipc_dir, AMEM_GROUPID=str(gid), AMEM_SLOT="1")
     from asystem_amem_amd import binding as B, harness as H
     from asystem_amem_amd.footprint import Footprint
-    lib = B.load()
+    lib = B.load(lib_path)
     lib.amem_set_option(b"peer_timeout_ms", 60000)     # the point: it must not take this long
     fp = Footprint(2, 32, max_regions=4, threads=2)
     regs = H.Regions(lib, fp)
