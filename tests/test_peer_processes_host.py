@@ -132,3 +132,109 @@ def test_importer_whose_owner_died_while_paused_gets_an_error_not_a_hang(standin
             for p in (owner, imp):
                 if p.is_alive():
                     p.kill()
+
+
+def _plain_owner(ipc_dir, gid, lib_path, conn, ctrl):
+    os.environ.update(AMEM_ENABLE="1", GMM_LOG="1", GMM_IPC_DIR=ipc_dir, AMEM_GROUPID=str(gid), AMEM_SLOT="0")
+    from asystem_amem_amd import binding as B, harness as H
+    from asystem_amem_amd.footprint import Footprint
+    lib = B.load(lib_path)
+    fp = Footprint(2, 33, max_regions=3, threads=2)
+    regs = H.Regions(lib, fp)
+    for i in range(3):
+        fd = C.c_int(-1)
+        assert lib.amem_vmm_export(int(regs.handle[i]), C.byref(fd)) == 0
+        conn.send((int(regs.handle[i]), int(regs.alloc[i])))
+        reduction.send_handle(conn, fd.value, None)
+        os.close(fd.value)
+    for cycle in range(2):
+        ctrl.send("ready"); assert ctrl.recv() == "pause"
+        assert lib.amem_mem_pause(0, 0) == 0
+        ctrl.send("paused"); assert ctrl.recv() == "resume"
+        assert lib.amem_mem_resume(0, 0) == 0
+        assert regs.mismatched_bytes() == 0
+        ctrl.send("resumed")
+    assert ctrl.recv() == "exit"
+    regs.free()
+    lib.amem_shutdown()
+
+
+def _importer_without_memory_of_its_own(ipc_dir, gid, lib_path, conn, ctrl):
+    os.environ.update(AMEM_ENABLE="1", GMM_LOG="1", GMM_IPC_DIR=ipc_dir, AMEM_GROUPID=str(gid), AMEM_SLOT="1")
+    from asystem_amem_amd import binding as B, harness as H
+    from asystem_amem_amd.footprint import Footprint
+    lib = B.load(lib_path)
+    fp = Footprint(2, 33, max_regions=3, threads=2)      # the owner's footprint, to check the bytes against
+    imported = []
+    for _ in range(3):
+        owner_handle, size = conn.recv()
+        fd = reduction.recv_handle(conn)
+        va, h = C.c_uint64(), C.c_uint64()
+        assert lib.amem_vmm_import(fd, size, 0, C.byref(va), C.byref(h)) == 0
+        os.close(fd)
+        assert lib.amem_add_alloc_info(va.value, size, B.TYPE_PEER_POSIX, 0, h.value, 0, owner_handle, None,
+                                       B.CALLER_P2P_PEER) == 0
+        imported.append((va.value, size))
+
+    def bad_bytes():
+        bad = 0
+        for i, (va, size) in enumerate(imported):
+            buf = np.empty(int(fp.sizes[i]), dtype=np.uint8)
+            assert lib.amem_copy_from_device(buf.ctypes.data, va, buf.nbytes) == 0
+            bad += fp.check_region(i, buf)
+        return bad
+
+    assert bad_bytes() == 0
+    for cycle in range(2):
+        ctrl.send("ready"); assert ctrl.recv() == "pause"
+        assert lib.amem_mem_pause(0, 0) == 0                 # nothing of its own to save: mappings dropped, nothing copied
+        c, st = H.counters(lib), H.cycle_stats(lib)
+        assert (c["offload_cnt"], c["release_shadow_cnt"], c["release_local_cnt"], c["paused"]) == (0, 3, 0, 1)
+        assert st["parked_bytes"] == 0 and st["local_regions"] == 0 and st["peer_regions"] == 3
+        ctrl.send("paused"); assert ctrl.recv() == "resume"
+        assert lib.amem_mem_resume(0, 0) == 0                # returns once the owner has re-exported all three
+        c = H.counters(lib)
+        assert (c["release_shadow_cnt"], c["paused"]) == (0, 0)
+        assert bad_bytes() == 0
+        ctrl.send("resumed")
+    assert ctrl.recv() == "exit"
+    for va, size in imported:
+        lib.amem_del_alloc_info(va, 0, 0)
+        lib.amem_vmm_free(va, size, 0)
+    lib.amem_shutdown()
+
+
+def test_process_that_only_imports(standin):
+    """A process whose whole registry is other processes' memory (an importer with no buffers of its own):
+    its pause has nothing to scan or copy and only drops mappings, its resume only waits for the owner."""
+    ctx = mp.get_context("spawn")
+    with tempfile.TemporaryDirectory() as ipc_dir:
+        gid = 0x6a00 + os.getpid() % 1024
+        a, b = ctx.Pipe(duplex=True)
+        oc, ic = ctx.Pipe(duplex=True), ctx.Pipe(duplex=True)
+        owner = ctx.Process(target=_plain_owner, args=(ipc_dir, gid, standin, a, oc[1]))
+        imp = ctx.Process(target=_importer_without_memory_of_its_own, args=(ipc_dir, gid, standin, b, ic[1]))
+        owner.start(); imp.start()
+        try:
+            for cycle in range(2):
+                for c in (oc[0], ic[0]):
+                    assert c.poll(60) and c.recv() == "ready"
+                ic[0].send("pause")
+                assert ic[0].poll(60) and ic[0].recv() == "paused"
+                oc[0].send("pause")
+                assert oc[0].poll(60) and oc[0].recv() == "paused"
+                # the importer resumes first in the second cycle and has to wait for the owner
+                first, second = (oc[0], ic[0]) if cycle == 0 else (ic[0], oc[0])
+                first.send("resume")
+                if cycle == 1:
+                    time.sleep(0.3)
+                second.send("resume")
+                for c in (oc[0], ic[0]):
+                    assert c.poll(60) and c.recv() == "resumed"
+            oc[0].send("exit"); ic[0].send("exit")
+            owner.join(30); imp.join(30)
+            assert owner.exitcode == 0 and imp.exitcode == 0
+        finally:
+            for p in (owner, imp):
+                if p.is_alive():
+                    p.kill()
