@@ -338,7 +338,7 @@ def test_failed_allocation_and_import_leave_nothing_behind(eng):
     os.close(r); os.close(w)
     assert lib.amem_vmm_import(r, 2 * MiB, 0, C.byref(iva), C.byref(ih)) != 0    # closed by now
     assert iva.value == 0 and ih.value == 0
-    assert H.mem_free(lib) == free0
+    assert abs(H.mem_free(lib) - free0) < MiB      # (every allocation here is 2 MiB or more)
     # an import that succeeds but cannot be mapped, because the address it is meant for still holds a
     # mapping: the reference taken by the import is dropped again, the descriptor is closed, the mapping
     # that was there is untouched
@@ -353,7 +353,7 @@ def test_failed_allocation_and_import_leave_nothing_behind(eng):
     fd = C.c_int(-1)
     assert lib.amem_vmm_export(b[1].value, C.byref(fd)) == 0
     assert lib.amem_update_peer_info(a[0].value, fd.value) != 0
-    assert len(os.listdir("/proc/self/fd")) == nfds and H.mem_free(lib) == free1
+    assert len(os.listdir("/proc/self/fd")) == nfds and abs(H.mem_free(lib) - free1) < MiB
     out = np.empty_like(data)
     assert lib.amem_copy_from_device(out.ctypes.data, a[0].value, out.nbytes) == 0 and np.array_equal(out, data)
     t = H.region_table(lib, 0)[a[0].value]
@@ -365,7 +365,7 @@ def test_failed_allocation_and_import_leave_nothing_behind(eng):
     free2 = H.mem_free(lib)
     assert lib.amem_vmm_alloc(8 * MiB, 0, C.byref(va), C.byref(h), C.byref(asz)) == 0
     assert lib.amem_vmm_free(va.value, asz.value, h.value) == 0
-    assert H.mem_free(lib) == free2
+    assert abs(H.mem_free(lib) - free2) < MiB
 
 
 def test_offload_free_tag_releases_without_copy(eng):
