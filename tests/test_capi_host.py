@@ -346,3 +346,22 @@ def test_offload_free_tag_variable_becomes_the_option():
             env["AMEM_NCCL_OFFLOAD_FREE_TAG"] = value
         out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, check=True).stdout
         assert ("tag %d" % want) in out, (value, out)
+
+
+def test_registry_latency_at_configuration_4_size(tmp_path):
+    """benchmark configuration 4 asks for registry latency: 100,000 entries (its sub-allocation count)
+    added through the hook in shuffled order, looked up by handle and by address, deleted. Reported per
+    call; the bound asserted here is loose (this is a shared CPU box), the figure goes into the output."""
+    libdir = os.path.dirname(B.LIB_PATH)
+    exe = str(tmp_path / "registry_latency")
+    subprocess.run(["g++", "-O2", "-std=c++17", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(ROOT, "include"),
+                    os.path.join(ROOT, "tests", "host_race", "registry_latency.cpp"), "-o", exe, B.LIB_PATH,
+                    "-Wl,-rpath," + libdir], check=True, capture_output=True, text=True)
+    env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="1", AMEM_IPC="0")
+    r = subprocess.run([exe, "100000"], env=env, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, (r.stdout[-2000:], r.stderr[-2000:])
+    line = [l for l in r.stdout.splitlines() if l.startswith("registry latency")][0]
+    print(line)
+    figures = [float(v) for v in re.findall(r"([0-9.]+) us", line)]
+    assert len(figures) == 5 and all(v < 50.0 for v in figures), line
+    assert "errors 0" in line
