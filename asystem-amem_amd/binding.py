@@ -57,7 +57,7 @@ class CycleStats(C.Structure):
         "k1_launches", "k2_launches", "k3_launches", "footprint_bytes", "parked_bytes", "zero_chunks",
         "total_chunks", "local_regions", "peer_regions", "dma_bytes", "kernel_bytes", "slab_bytes",
         "verify_mismatch")] + [(n, C.c_double) for n in (
-        "pause_pool_ms", "pause_scratch_ms", "pause_sync_ms", "resume_scratch_ms")]
+        "pause_pool_ms", "pause_scratch_ms", "pause_sync_ms", "resume_scratch_ms")] + [("resume_dma_bytes", C.c_uint64)]
 
     def as_dict(self):
         return {k: getattr(self, k) for k, _ in self._fields_}
@@ -117,6 +117,8 @@ _SIGNATURES = {
     "amem_get_slot": (C.c_int, []),
     "amem_ipc_claim_slot": (C.c_int, []),
     "amem_ipc_act_as": (C.c_int, [C.c_int]),
+    "amem_ipc_served": (C.c_int, [C.c_int, C.POINTER(C.c_uint64)]),
+    "amem_ipc_peer_alive": (C.c_int, [C.c_int]),
     "amem_chunk_count": (C.c_uint64, [C.POINTER(Extent), C.c_uint64]),
     "amem_zero_scan": (C.c_int, [C.POINTER(Extent), C.c_uint64, C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
     "amem_zero_scan_noalloc": (C.c_int, [C.POINTER(Extent), C.c_uint64, C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),

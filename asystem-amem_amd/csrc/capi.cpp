@@ -312,14 +312,21 @@ int amem_register_peer_info(uint64_t src_handle, uint64_t peer_va, int peer_dev)
     std::lock_guard<std::mutex> lf(c->fields);
     for (int dev = 0; dev < AMEM_MAX_DEVS && ret; ++dev) {
       auto ht = c->handleTable[dev].find(src_handle);
-      if (ht == c->handleTable[dev].end()) continue;
-      auto it = c->allocTable[dev].find(ht->second);
+      auto it = c->allocTable[dev].end();
+      if (ht != c->handleTable[dev].end()) {
+        it = c->allocTable[dev].find(ht->second);
+      } else {
+        // Not a handle of this process: an importer that cannot know the current handle value (it changes
+        // with every resume) may name the region by the owner's address instead, which never changes.
+        it = c->allocTable[dev].find(src_handle);
+        if (it != c->allocTable[dev].end() && from_peer(it->second.type)) it = c->allocTable[dev].end();
+      }
       if (it == c->allocTable[dev].end()) continue;
       it->second.peers[peer_dev] = peer_va;
       it->second.hasPeer = true;
       ret = 0;
       LOGGER(DEBUG, "groupID:%d pid:%d localDptr:%llx localHandle:%llx register peer:%d peerPtr:%llx done",
-             amem_groupID, getpid(), (unsigned long long)ht->second, (unsigned long long)src_handle, peer_dev,
+             amem_groupID, getpid(), (unsigned long long)it->first, (unsigned long long)src_handle, peer_dev,
              (unsigned long long)peer_va);
     }
   }
@@ -335,7 +342,12 @@ int amem_update_peer_info(uint64_t va, int shared_fd) {
   int dev = -1;
   size_t size = 0;
   int state = AMEM_STATE_INVALID;
+  const bool gpu = gpu_present();
   {
+    // Only an address that a pause has emptied can take new memory. The CUDA driver refuses to map
+    // over an existing mapping; this HIP runtime accepts it (measured) and the old mapping would be
+    // lost without being unmapped. So the hole is claimed here, under the lock: of two updates for one
+    // address (a retried owner resume, two service threads of one process) the second finds it taken.
     std::lock_guard<std::mutex> lf(c->fields);
     for (int d = 0; d < AMEM_MAX_DEVS && dev < 0; ++d) {
       auto it = c->allocTable[d].find(va);
@@ -343,6 +355,7 @@ int amem_update_peer_info(uint64_t va, int shared_fd) {
       dev = d;
       size = it->second.allocSz;
       state = it->second.state;
+      if (state == AMEM_STATE_HOLE && gpu) it->second.state = AMEM_STATE_PRELOADING;
     }
   }
   if (dev < 0) {
@@ -351,35 +364,39 @@ int amem_update_peer_info(uint64_t va, int shared_fd) {
     if (shared_fd >= 0) close(shared_fd);
     return 1;
   }
-  // Only an address that a pause has emptied can take new memory. The CUDA driver refuses to map
-  // over an existing mapping; this HIP runtime accepts it (measured) and the old mapping would be
-  // lost without being unmapped, so the state is checked here.
   if (state != AMEM_STATE_HOLE) {
     LOGGER(ERROR, "groupID:%d pid:%d dptr:%llx is not released (state %d): refusing to map fd:%d over it", amem_groupID,
            getpid(), (unsigned long long)va, state, shared_fd);
     if (shared_fd >= 0) close(shared_fd);
     return 1;
   }
-  if (!gpu_present()) {
+  if (!gpu) {
     LOGGER(ERROR, "pid:%d no HIP device: cannot import fd:%d", getpid(), shared_fd);
     close(shared_fd);
     return 1;
   }
   uint64_t newh = 0;
   int ret = (int)vmm_import_map(dev, va, size, shared_fd, true, &newh);  // amem_importAndMap
-  if (ret == 0) {
+  {
     std::lock_guard<std::mutex> lf(c->fields);
     auto it = c->allocTable[dev].find(va);
-    if (it != c->allocTable[dev].end()) {
-      it->second.state = AMEM_STATE_ALLOC;
-      it->second.handle = newh;
-      it->second.handleGen++;
+    if (it != c->allocTable[dev].end() && it->second.state == AMEM_STATE_PRELOADING) {
+      if (ret == 0) {
+        it->second.state = AMEM_STATE_ALLOC;
+        it->second.handle = newh;
+        it->second.handleGen++;
+      } else {
+        it->second.state = AMEM_STATE_HOLE;  // nothing is mapped: a later update may try again
+      }
     }
-    c->releaseShadowCnt--;
-    c->shadow_cv.notify_all();
+    if (ret == 0) {
+      c->releaseShadowCnt--;
+      c->shadow_cv.notify_all();
+    }
+  }
+  if (ret == 0)
     LOGGER(DEBUG, "groupID:%d pid:%d curDev:%d update ptr:%llx fd:%d done", amem_groupID, getpid(), dev,
            (unsigned long long)va, shared_fd);
-  }
   return ret;
 }
 
@@ -708,6 +725,8 @@ int amem_ipc_claim_slot(void) {
   return ipc_claim_extra();
 }
 int amem_ipc_act_as(int slot) { return ipc_act_as(slot); }
+int amem_ipc_served(int slot, uint64_t counts[3]) { return counts ? ipc_served(slot, counts) : 1; }
+int amem_ipc_peer_alive(int slot) { return peer_alive(slot) ? 1 : 0; }
 
 // ---- kernels on their own ----
 
@@ -812,10 +831,24 @@ static void __attribute__((constructor)) amem_lib_init(void) {
   amem_groupID = getenv("AMEM_GROUPID") ? atoi(getenv("AMEM_GROUPID")) : 0;
   int cuMemFlag = getenv("NCCL_CUMEM_ENABLE") ? atoi(getenv("NCCL_CUMEM_ENABLE")) : 1;
   if (cuMemFlag == 0) g.disabled = 1;
-  // The reference parses the tag (amem_nccl.cpp:478, :587) and then compares against a macro, so
-  // the variable never acts there; here it selects the caller tag whose regions are released
-  // without being copied, which is what its README documents (README.md:224, run.sh:9-18).
-  if (g.offload_free_tag >= 0 && g.offload_free_tag < AMEM_MAX_CALLER) options().offload_free_tag = g.offload_free_tag;
+  // The reference parses the tag (amem_nccl.cpp:478, :587) and then compares against a macro, so the
+  // variable never acts there and regions of every tag keep their bytes. By default this library
+  // does the same. With AMEM_OFFLOAD_FREE_TAG_APPLY=1 the variable takes effect: it selects the
+  // caller tag whose regions are released without being copied and come back zero-filled, which is
+  // what the reference's README documents (README.md:224, run.sh:9-18).
+  const bool apply_tag = getenv("AMEM_OFFLOAD_FREE_TAG_APPLY") && atoi(getenv("AMEM_OFFLOAD_FREE_TAG_APPLY")) != 0;
+  if (g.offload_free_tag >= 0 && g.offload_free_tag < AMEM_MAX_CALLER) {
+    if (apply_tag) {
+      options().offload_free_tag = g.offload_free_tag;
+      LOGGER(WARN, "groupID:%d pid:%d AMEM_NCCL_OFFLOAD_FREE_TAG=%d is applied: regions registered with caller tag %d "
+             "are released without a copy and come back ZERO-FILLED after resume (the reference keeps their bytes)",
+             amem_groupID, getpid(), g.offload_free_tag, g.offload_free_tag);
+    } else if (!g.disabled) {
+      LOGGER(INFO, "groupID:%d pid:%d AMEM_NCCL_OFFLOAD_FREE_TAG=%d is read but not applied, as in the reference "
+             "(regions of every tag keep their bytes); set AMEM_OFFLOAD_FREE_TAG_APPLY=1 to release regions of that "
+             "tag without a copy", amem_groupID, getpid(), g.offload_free_tag);
+    }
+  }
   LOGGER(INFO, "groupID:%d pid:%d build:%s %s NCCL plugin loaded. pause func:%s offload_free_tag:%d cuMemEnabled:%d",
          amem_groupID, getpid(), __DATE__, __TIME__, g.disabled ? "Off" : "On", g.offload_free_tag, cuMemFlag);
 }

@@ -1062,7 +1062,7 @@ int Engine::resume(Ctx& c, bool* incomplete) {
          (long)((total - free_sz) >> 20));
   auto t0 = Clock::now();
   stats_.resume_ms = stats_.resume_map_ms = stats_.resume_copy_ms = stats_.resume_peer_ms = 0;
-  stats_.k3_ms = 0; stats_.k3_launches = 0; stats_.verify_mismatch = 0;
+  stats_.k3_ms = 0; stats_.k3_launches = 0; stats_.verify_mismatch = 0; stats_.resume_dma_bytes = 0;
   (void)take_scratch_alloc_ms();
   auto& table = c.allocTable[dev_];
 
@@ -1132,7 +1132,10 @@ int Engine::resume(Ctx& c, bool* incomplete) {
   const uint64_t* tp = (const uint64_t*)h_tiles_.p;
   SlabTable pool_tab = {(uint8_t* const*)d_slabtab_.p, pool_->shift(), pool_->slab_bytes() - 1};
 
-  struct Export { Region* r; uint64_t va; int fd; };
+  // Regions whose new memory has importers. Each is exported only when its importers are told
+  // (below), so that one descriptor is open at a time, as in the reference's loop
+  // (amem_nccl.cpp:613, :646), however many regions there are.
+  struct Export { Region* r; uint64_t va; uint64_t handle; };
   std::vector<Export> exports;
   uint64_t exportSz = 0;
   size_t ev = 8;
@@ -1164,9 +1167,7 @@ int Engine::resume(Ctx& c, bool* incomplete) {
         c.handleTable[dev_].emplace(newh, im.va);
       }
       if (has_peer) {
-        int fd = -1;
-        note(vmm_export_fd(newh, &fd));
-        exports.push_back({im.r, im.va, fd});
+        exports.push_back({im.r, im.va, newh});
         exportSz += im.r->allocSz;
       }
       if (ref_mode_) {
@@ -1182,7 +1183,7 @@ int Engine::resume(Ctx& c, bool* incomplete) {
       for (uint32_t m = im.m0; m < im.m1 && rc == 0; ++m) {
         note(CHECK_HIP(hipMemcpyAsync((void*)(uintptr_t)dma[m].va, pool_->host_addr(dma[m].off), dma[m].bytes,
                                       hipMemcpyHostToDevice, dstream_)));
-        stats_.dma_bytes += dma[m].bytes;
+        stats_.resume_dma_bytes += dma[m].bytes;
       }
       bytes += im.bytes;
       ++j;
@@ -1249,9 +1250,13 @@ int Engine::resume(Ctx& c, bool* incomplete) {
       std::lock_guard<std::mutex> lk(c.fields);
       memcpy(peers, x.r->peers, sizeof(peers));
     }
+    int fd = -1;
+    e = vmm_export_fd(x.handle, &fd);
+    note(e);
+    if (e != hipSuccess) continue;
     for (int s = 0; s < AMEM_MAX_DEVS; ++s) {
       if (peers[s] == 0) continue;
-      int ret = peer_update(s, peers[s], x.fd);
+      int ret = peer_update(s, peers[s], fd);
       if (ret != 0 && !peer_alive(s)) {
         // The importer's process is gone and its mapping with it: nothing to update, now or later.
         LOGGER(WARN, "groupID:%d pid:%d localDptr:%llx the importer in slot %d is gone, forgetting its mapping %llx",
@@ -1263,7 +1268,7 @@ int Engine::resume(Ctx& c, bool* incomplete) {
         c.releaseLocalCnt--;
       } else if (ret != 0) {
         LOGGER(ERROR, "groupID:%d pid:%d localDptr:%llx newHandle:%llx fd:%d notify peer %d to remap dptr:%llx ret:%d",
-               amem_groupID_value(), getpid(), (unsigned long long)x.va, (unsigned long long)x.r->handle, x.fd,
+               amem_groupID_value(), getpid(), (unsigned long long)x.va, (unsigned long long)x.handle, fd,
                s, (unsigned long long)peers[s], ret);
         if (rc == 0) rc = ret;
       } else {
@@ -1271,7 +1276,7 @@ int Engine::resume(Ctx& c, bool* incomplete) {
         c.releaseLocalCnt--;
       }
     }
-    if (x.fd >= 0) close(x.fd);
+    if (fd >= 0) close(fd);
   }
 
   // Wait until every mapping this process imports has been re-established by its owner

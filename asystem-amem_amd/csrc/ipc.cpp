@@ -57,6 +57,8 @@ struct Service {
   std::string sock_path, lock_path;
   std::thread thr;
   std::atomic<bool> stop{false};
+  std::atomic<uint64_t> served[3];  // requests answered with success: register, update, release
+  Service() { for (auto& n : served) n.store(0); }
 };
 // A process normally holds one slot (`primary`). It may claim more, one per rank it hosts: each
 // extra slot is a full peer with a lock, a socket and a service thread of its own, so that ranks
@@ -213,6 +215,8 @@ void serve(Service* svc_p) {
         continue;
       }
       int32_t ret = handle_request(req, fd);
+      if (ret == 0 && req.op >= OP_REGISTER_PEER_INFO && req.op <= OP_RELEASE_PEER_HANDLE)
+        g_svc.served[req.op - OP_REGISTER_PEER_INFO].fetch_add(1, std::memory_order_relaxed);
       send_msg(fds[i].fd, &ret, sizeof(ret), -1);
       ++i;
     }
@@ -344,6 +348,7 @@ static bool start_service(Service& svc) {
     return false;
   }
   svc.stop.store(false);
+  for (auto& n : svc.served) n.store(0);
   svc.thr = std::thread(serve, &svc);
   LOGGER(DEBUG, "groupID:%d pid:%d serving slot %d on %s", amem_groupID_value(), getpid(), svc.slot,
          svc.sock_path.c_str());
@@ -402,6 +407,15 @@ int ipc_claim_extra() {
   }
   g_ipc.extra.push_back(svc);
   return svc->slot;
+}
+
+int ipc_served(int slot, uint64_t out[3]) {
+  std::lock_guard<std::mutex> lk(g_ipc.mtx);
+  Service* svc = g_svc.slot == slot && slot >= 0 ? &g_svc : nullptr;
+  for (Service* s : g_ipc.extra) if (s->slot == slot) svc = s;
+  if (!svc) return 1;
+  for (int i = 0; i < 3; ++i) out[i] = svc->served[i].load(std::memory_order_relaxed);
+  return 0;
 }
 
 int ipc_act_as(int slot) {

@@ -24,6 +24,10 @@ int ipc_claim_extra();
 // From now on this thread registers imported regions as `slot` (one of this process's own; -1 =
 // the primary slot again). 0 ok, 1 when the process does not hold that slot.
 int ipc_act_as(int slot);
+// How many requests the service of this process's `slot` has answered with success since it
+// started: out[0] registrations, out[1] re-exported descriptors mapped, out[2] release requests.
+// 0 ok, 1 when the process does not hold that slot.
+int ipc_served(int slot, uint64_t out[3]);
 void ipc_stop();
 int ipc_slot();
 // Whether a process currently holds `slot` of this group (a crashed one no longer does).

@@ -251,7 +251,7 @@ typedef struct amem_cycle_stats {
   uint64_t parked_bytes;    /* bytes that crossed the host link per leg */
   uint64_t zero_chunks, total_chunks;
   uint64_t local_regions, peer_regions;
-  uint64_t dma_bytes;       /* of parked_bytes, how much moved by hipMemcpyAsync */
+  uint64_t dma_bytes;       /* of parked_bytes, how much the pause moved by hipMemcpyAsync */
   uint64_t kernel_bytes;    /* of parked_bytes, how much moved by the pack/unpack kernels */
   uint64_t slab_bytes;      /* pinned host memory held by the pool */
   uint64_t verify_mismatch; /* chunks whose checksum differed after resume (verify mode) */
@@ -259,6 +259,7 @@ typedef struct amem_cycle_stats {
   double pause_scratch_ms;  /* of pause_ms: allocating or growing the engine's own tables, staging and events */
   double pause_sync_ms;     /* of pause_ms: the device synchronisation and memory queries before the scan */
   double resume_scratch_ms; /* of resume_ms: allocating or growing the engine's own tables and events */
+  uint64_t resume_dma_bytes; /* of parked_bytes, how much the resume brought back by hipMemcpyAsync */
 } amem_cycle_stats;
 void amem_get_cycle_stats(amem_cycle_stats* out);
 
@@ -304,9 +305,10 @@ int amem_set_enabled(int on);
  *   "offload_free_tag" caller tag (0-15, -1 = none) whose regions hold scratch data: pause releases
  *                     them without copying and resume hands them back zero-filled. This is what
  *                     AMEM_NCCL_OFFLOAD_FREE_TAG is documented to do in the reference, where the
- *                     variable is parsed but never takes effect (amem_nccl.cpp:40, :503, :620).
- *                     Here the variable, read when the library is loaded, is this option's
- *                     initial value
+ *                     variable is parsed but never takes effect (amem_nccl.cpp:40, :503, :620) and
+ *                     regions of every tag keep their bytes. The variable alone changes nothing
+ *                     here either; together with AMEM_OFFLOAD_FREE_TAG_APPLY=1 it becomes this
+ *                     option's initial value when the library is loaded (a WARN line says so)
  *   "release_thread"  0/1 (default 1): the default pause path releases handles on a thread of their own
  *                     instead of on the one that unmaps
  *   "scratch_on_host" 0/1: keep the engine's own tables in pinned host memory. That is where they go
@@ -335,7 +337,8 @@ int amem_shutdown(void);
 /* Slot of this process within its group on this node: index into peers[] that importers
  * pass as `peer_dev`. Taken from AMEM_SLOT or claimed first-free when the IPC service
  * starts. Returns -1 before that. amem_ipc_start starts the service explicitly (it is
- * otherwise started by the first add of a peer-type region or by amem_get_slot). */
+ * otherwise started together with the context, by the first tracked allocation, unless
+ * AMEM_IPC=0) and returns the slot. */
 int amem_ipc_start(void);
 int amem_get_slot(void);
 /* A process that hosts several ranks gives each of them a slot of its own: amem_ipc_claim_slot
@@ -349,6 +352,13 @@ int amem_get_slot(void);
  * one worker per (process, GPU). */
 int amem_ipc_claim_slot(void);
 int amem_ipc_act_as(int slot);
+/* What the service of this process's `slot` has answered with success since it started:
+ * counts[0] registrations of an importer (gmm_worker_impl.cpp:375-382), counts[1] re-exported
+ * descriptors mapped at an importer's address (:384-390), counts[2] release requests (:392-397).
+ * 0 ok, 1 when this process does not hold `slot`. Inspection only. */
+int amem_ipc_served(int slot, uint64_t counts[3]);
+/* 1 while some process holds `slot` of this group on this node (its lock dies with it), else 0. */
+int amem_ipc_peer_alive(int slot);
 
 /* ---------------------------------------------------------------------------------------
  * 6. The device kernels, callable on their own (no reference counterpart: the reference

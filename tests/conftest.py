@@ -17,6 +17,23 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+_MEASURED = []
+
+
+@pytest.fixture()
+def measured():
+    """Tests hand timings here (one line each); they are printed in the run's summary, where `-q` and
+    output capture do not hide them."""
+    return _MEASURED.append
+
+
+def pytest_terminal_summary(terminalreporter):
+    if _MEASURED:
+        terminalreporter.section("measured")
+        for line in _MEASURED:
+            terminalreporter.write_line(line)
+
+
 def _built():
     from asystem_amem_amd import binding, footprint
     import oracle

@@ -14,17 +14,19 @@ from multiprocessing import reduction
 import numpy as np
 
 MiB = 1 << 20
-NREG = 6          # regions per process (config-2 distribution: 4 MiB channel buffers first)
+NREG = 6          # default regions per process (config-2 distribution: 4 MiB channel buffers first); 256 = all of it
 
 
 def _nfds():
     return len(os.listdir("/proc/self/fd"))
 
 
-def _worker(rank, world, ipc_dir, gid, conns, ctrl, lib_path=None):
+def _worker(rank, world, ipc_dir, gid, conns, ctrl, lib_path=None, NREG=NREG):
     """conns[j]: duplex connection to rank j (None for self); ctrl: connection to the parent;
-    lib_path: library to load instead of the shipped one (the host stand-in build)."""
+    lib_path: library to load instead of the shipped one (the host stand-in build);
+    NREG: regions this process owns (and imports from every peer)."""
     try:
+        import threading
         os.environ.update(AMEM_ENABLE="1", GMM_LOG="2", GMM_IPC_DIR=ipc_dir, AMEM_GROUPID=str(gid), AMEM_SLOT=str(rank))
         from asystem_amem_amd import binding as B, harness as H
         from asystem_amem_amd.footprint import Footprint
@@ -34,16 +36,20 @@ def _worker(rank, world, ipc_dir, gid, conns, ctrl, lib_path=None):
         regs = H.Regions(lib, fp)                      # local regions, registered
         assert lib.amem_get_slot() == rank
         ctrl.send(("ready", rank)); assert ctrl.recv() == "go"
-        # export to every peer
-        for j in range(world):
-            if j == rank:
-                continue
-            for i in range(NREG):
-                fd = C.c_int(-1)
-                assert lib.amem_vmm_export(int(regs.handle[i]), C.byref(fd)) == 0
-                conns[j].send((i, int(regs.handle[i]), int(regs.alloc[i])))
-                reduction.send_handle(conns[j], fd.value, None)
-                os.close(fd.value)
+        # export to every peer; on a thread of its own, so that with hundreds of regions two processes
+        # that both have a full socket towards each other still drain what the other one sends
+        def export_all():
+            for j in range(world):
+                if j == rank:
+                    continue
+                for i in range(NREG):
+                    fd = C.c_int(-1)
+                    assert lib.amem_vmm_export(int(regs.handle[i]), C.byref(fd)) == 0
+                    conns[j].send((i, int(regs.handle[i]), int(regs.alloc[i])))
+                    reduction.send_handle(conns[j], fd.value, None)
+                    os.close(fd.value)
+        exporter = threading.Thread(target=export_all)
+        exporter.start()
         # import from every peer and register with the owner
         imported = {}   # (owner, i) -> (va, size)
         for j in range(world):
@@ -59,6 +65,8 @@ def _worker(rank, world, ipc_dir, gid, conns, ctrl, lib_path=None):
                                              B.CALLER_P2P_PEER)
                 assert rc == 0, ("register with owner failed", rank, j, i, rc)
                 imported[(j, i)] = (va.value, size)
+        exporter.join()
+        assert len(imported) == NREG * (world - 1)
         ctrl.send(("imported", rank)); assert ctrl.recv() == "go"
         peers_fp = {j: Footprint(2, 4 + j, max_regions=NREG, threads=2) for j in range(world) if j != rank}
 
@@ -128,9 +136,9 @@ def _worker(rank, world, ipc_dir, gid, conns, ctrl, lib_path=None):
 
 
 
-def run_world(world, lib_path=None, gid_base=0x6000):
-    """Start `world` worker processes, walk them through the phases in lock step, and insist that every
-    one of them finishes cleanly."""
+def run_world(world, lib_path=None, gid_base=0x6000, nreg=NREG, phase_timeout=120):
+    """Start `world` worker processes, each owning `nreg` regions, walk them through the phases in lock
+    step, and insist that every one of them finishes cleanly."""
     ctx = mp.get_context("spawn")
     with tempfile.TemporaryDirectory() as ipc_dir:
         gid = gid_base + os.getpid() % 4096 + world
@@ -142,14 +150,14 @@ def run_world(world, lib_path=None, gid_base=0x6000):
         procs = []
         for r in range(world):
             conns = [pair.get((r, j)) for j in range(world)]
-            p = ctx.Process(target=_worker, args=(r, world, ipc_dir, gid, conns, ctrls[r][1], lib_path))
+            p = ctx.Process(target=_worker, args=(r, world, ipc_dir, gid, conns, ctrls[r][1], lib_path, nreg))
             p.start()
             procs.append(p)
         try:
             phases = ["ready", "imported", "checked"] + ["paused", "freed", "resumed", "verified"] * 2 + ["tagged", "done"]
             for phase in phases:
                 for r in range(world):
-                    assert ctrls[r][0].poll(120), "rank %d did not reach %s" % (r, phase)
+                    assert ctrls[r][0].poll(phase_timeout), "rank %d did not reach %s" % (r, phase)
                     msg = ctrls[r][0].recv()
                     assert msg[0] == phase, msg
                 for r in range(world):

@@ -332,20 +332,30 @@ def test_random_registry_sequences_match_oracle(fresh, fresh_orc, seed):
     p.check()
 
 
-def test_offload_free_tag_variable_becomes_the_option():
-    """AMEM_NCCL_OFFLOAD_FREE_TAG is read once, when the library is loaded (amem_nccl.cpp:478 reads it
-    per pause and never applies it); a valid tag becomes the engine's offload_free_tag option, anything
-    else leaves it off. run.sh of the reference sets 7."""
+def test_offload_free_tag_variable_becomes_the_option_only_when_asked_to():
+    """AMEM_NCCL_OFFLOAD_FREE_TAG is read once, when the library is loaded. The reference reads it per
+    pause and never applies it (amem_nccl.cpp:478 against the macro at :503, :620): regions of every tag
+    keep their bytes. By default this library does the same and says so; with AMEM_OFFLOAD_FREE_TAG_APPLY=1
+    a valid tag becomes the engine's offload_free_tag option (and a WARN line names what that means),
+    anything else leaves it off. run.sh of the reference sets 7."""
     code = ("import sys; sys.path.insert(0, %r)\n"
             "from asystem_amem_amd import binding as B\n"
             "print('tag', B.load().amem_get_option(b'offload_free_tag'))\n" % ROOT)
-    for value, want in (("7", 7), ("0", 0), ("15", 15), ("16", -1), ("-3", -1), (None, -1)):
-        env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="1", AMEM_IPC="0")
+    for value, apply, want in (("7", "1", 7), ("0", "1", 0), ("15", "1", 15), ("16", "1", -1), ("-3", "1", -1),
+                               (None, "1", -1), ("7", None, -1), ("7", "0", -1)):
+        env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="3", AMEM_IPC="0")
         env.pop("AMEM_NCCL_OFFLOAD_FREE_TAG", None)
+        env.pop("AMEM_OFFLOAD_FREE_TAG_APPLY", None)
         if value is not None:
             env["AMEM_NCCL_OFFLOAD_FREE_TAG"] = value
+        if apply is not None:
+            env["AMEM_OFFLOAD_FREE_TAG_APPLY"] = apply
         out = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, check=True).stdout
-        assert ("tag %d" % want) in out, (value, out)
+        assert ("tag %d" % want) in out, (value, apply, out)
+        if value == "7":
+            assert "offload_free_tag:7" in out                       # the load line reports what was read, as the reference's does
+            assert ("ZERO-FILLED" in out) == (want == 7)
+            assert ("read but not applied" in out) == (want != 7)
 
 
 def test_registry_latency_at_configuration_4_size(tmp_path):

@@ -226,7 +226,7 @@ def test_owner_forgets_an_importer_whose_process_is_gone(gpu, fresh):
 
 
 
-def test_config5_shape_three_importer_ranks_in_one_process(gpu, fresh):
+def test_config5_shape_three_importer_ranks_in_one_process(gpu, fresh, measured):
     """Benchmark configuration 5 at its full per-process shape, in the one form this machine's runtime
     allows (it refuses a VMM descriptor exported by another process): the process holds four slots, each
     with its own lock, socket and service thread; the first owns the 256 regions of configuration 2's
@@ -301,8 +301,8 @@ def test_config5_shape_three_importer_ranks_in_one_process(gpu, fresh):
         after = H.region_table(lib, 0)
         assert [d for d in H.compare_tables(before, after) if d[1] != "handle_gen"] == []
         assert all(after[va]["handle_gen"] == before[va]["handle_gen"] + 3 for va in before)   # three cycles, three new handles each
-        print("config-5 shape, one process: %d regions x %d importers, pause/resume/peer ms per cycle: %s" %
-              (N, R, ", ".join("%.0f/%.0f/%.0f" % t for t in times)))
+        measured("config-5 shape, one owner: %d regions x %d importers, pause/resume/peer ms per cycle: %s" %
+                 (N, R, ", ".join("%.0f/%.0f/%.0f" % t for t in times)))
         # one physical memory behind all four addresses of a region
         tag = np.full(4096, 0xC3, dtype=np.uint8)
         assert lib.amem_copy_to_device(int(regs.va[5]), tag.ctypes.data, 4096) == 0
@@ -314,6 +314,126 @@ def test_config5_shape_three_importer_ranks_in_one_process(gpu, fresh):
             lib.amem_del_alloc_info(va, 0, 0)
             lib.amem_vmm_free(va, int(regs.alloc[i]), 0)
         regs.free()
+    finally:
+        lib.amem_mem_resume(0, 0)
+        lib.amem_ipc_act_as(-1)
+        assert lib.amem_set_option(b"peer_loopback", 0) == 0
+
+
+def test_config5_every_rank_owns_and_imports_in_one_process(gpu, fresh, measured):
+    """Benchmark configuration 5's full matrix in the one form this machine's runtime allows (one process):
+    four slots, each with its own lock, socket and service thread; EVERY slot owns the 256 regions of
+    configuration 2's layout (seeds 4, 5, 6, 7: 4 x 1,216 MiB) and imports the 768 regions of the other
+    three at addresses of its own. 1,024 owned + 3,072 imported mappings; 3,072 registration requests spread
+    over four services; per resume 3,072 descriptor messages (SCM_RIGHTS), each owner's regions going to
+    three different services while the same process's services map what the other owners send. Closed forms
+    (amem_nccl.cpp:511 one offload per local region, :524 one releasePeer per imported mapping, :547-550 one
+    releaseLocal per recorded importer): 1,024 / 3,072 / 3,072 at pause, 0 / 0 / 0 after resume."""
+    from asystem_amem_amd import binding as B, harness as H
+    from asystem_amem_amd.footprint import Footprint
+    lib = fresh
+    assert lib.amem_set_option(b"peer_loopback", 1) == 0
+    try:
+        N, W = 256, 4
+        slots = [lib.amem_ipc_start()] + [lib.amem_ipc_claim_slot() for _ in range(W - 1)]
+        assert min(slots) >= 0 and len(set(slots)) == W
+        fps = [Footprint(2, 4 + k, max_regions=N, threads=8) for k in range(W)]
+        owned = [H.Regions(lib, fp) for fp in fps]          # rank k's own regions (local memory has no slot of its own)
+        assert all(len(r.va) == N and fp.total_bytes == 1216 * MiB for r, fp in zip(owned, fps))
+        total = sum(fp.total_bytes for fp in fps)
+        imports = {}                                         # (importing rank, owning rank, region) -> importer's address
+        for k in range(W):                                   # rank k imports from every other rank j
+            assert lib.amem_ipc_act_as(slots[k]) == 0
+            for j in range(W):
+                if j == k:
+                    continue
+                for i in range(N):
+                    fd, va, h = C.c_int(-1), C.c_uint64(), C.c_uint64()
+                    assert lib.amem_vmm_export(int(owned[j].handle[i]), C.byref(fd)) == 0
+                    assert lib.amem_vmm_import(fd.value, int(owned[j].alloc[i]), 0, C.byref(va), C.byref(h)) == 0
+                    os.close(fd.value)
+                    assert lib.amem_add_alloc_info(va.value, int(owned[j].alloc[i]), B.TYPE_PEER_POSIX, 0, h.value,
+                                                   slots[j], int(owned[j].handle[i]), None, B.CALLER_P2P_PEER) == 0
+                    imports[(k, j, i)] = va.value
+        assert lib.amem_ipc_act_as(-1) == 0
+        assert len(set(imports.values())) == W * (W - 1) * N
+
+        def imports_match():
+            bad = 0
+            buf = np.empty(max(int(fp.sizes.max()) for fp in fps), dtype=np.uint8)
+            for (k, j, i), va in imports.items():
+                n = int(fps[j].sizes[i])
+                assert lib.amem_copy_from_device(buf.ctypes.data, va, n) == 0
+                bad += fps[j].check_region(i, buf[:n])
+            return bad
+
+        def owned_match():
+            return sum(r.mismatched_bytes() for r in owned)
+
+        tab = H.region_table(lib, 0)
+        assert len(tab) == W * N + W * (W - 1) * N == 4096
+        for j in range(W):                                   # every owned region names exactly the three other slots
+            for i in range(N):
+                t = tab[int(owned[j].va[i])]
+                assert t["has_peer"] == 1
+                assert {s: p for s, p in enumerate(t["peers"]) if p} == \
+                    {slots[k]: imports[(k, j, i)] for k in range(W) if k != j}
+        assert all(tab[va]["type"] == B.TYPE_PEER_POSIX for va in imports.values())
+
+        def served():
+            out = {}
+            for s in slots:
+                n = (C.c_uint64 * 3)()
+                assert lib.amem_ipc_served(s, n) == 0
+                out[s] = tuple(n)
+            return out
+
+        # every owner's service took the registrations of the three other ranks, nobody else's
+        assert served() == {s: ((W - 1) * N, 0, 0) for s in slots}
+        c = H.counters(lib)
+        assert c["alloc_bytes"][B.CALLER_P2P] == total and c["alloc_bytes"][B.CALLER_P2P_PEER] == (W - 1) * total
+        assert owned_match() == 0 and imports_match() == 0
+        before = H.region_table(lib, 0)
+        assert lib.amem_mem_pause(0, 0) == 0 and lib.amem_mem_resume(0, 0) == 0     # warm cycle: engine scratch, pinned pool
+        fds0, free0 = _nfds(), H.mem_free(lib)
+        times = []
+        for cycle in range(2):
+            assert lib.amem_mem_pause(0, 0) == 0
+            c = H.counters(lib)
+            assert (c["offload_cnt"], c["release_shadow_cnt"], c["release_local_cnt"]) == \
+                (W * N, W * (W - 1) * N, W * (W - 1) * N) == (1024, 3072, 3072)
+            assert H.mem_free(lib) - free0 >= total - 16 * MiB   # all four references to every region are gone
+            assert all(t["state"] == B.STATE_HOLE for t in H.region_table(lib, 0).values())
+            assert lib.amem_check_paused(0) == 1
+            assert lib.amem_mem_resume(0, 0) == 0
+            st = H.cycle_stats(lib)
+            times.append((st["pause_ms"], st["resume_ms"], st["resume_peer_ms"]))
+            c = H.counters(lib)
+            assert (c["offload_cnt"], c["release_shadow_cnt"], c["release_local_cnt"], c["paused"]) == (0, 0, 0, 0)
+            assert _nfds() == fds0                           # 1,024 exported and 3,072 received descriptors, all closed
+            # every rank's service mapped the 768 descriptors the three other owners sent it (warm cycle included)
+            assert served() == {s: ((W - 1) * N, (cycle + 2) * (W - 1) * N, 0) for s in slots}
+            assert owned_match() == 0                        # 1,024 owner addresses against the four seeds
+            assert imports_match() == 0                      # and all 3,072 importer addresses
+        after = H.region_table(lib, 0)
+        assert [d for d in H.compare_tables(before, after) if d[1] != "handle_gen"] == []
+        assert all(after[va]["handle_gen"] == before[va]["handle_gen"] + 3 for va in before)
+        measured("config-5 matrix, one process: %d ranks x %d regions, each imported by %d: pause/resume/peer ms per cycle: %s" %
+                 (W, N, W - 1, ", ".join("%.0f/%.0f/%.0f" % t for t in times)))
+        # one physical memory behind all four addresses of a region, for a region of every owner
+        for j in range(W):
+            tag = np.full(4096, 0xC0 + j, dtype=np.uint8)
+            assert lib.amem_copy_to_device(int(owned[j].va[7]), tag.ctypes.data, 4096) == 0
+            for k in range(W):
+                if k != j:
+                    buf = np.empty(4096, dtype=np.uint8)
+                    assert lib.amem_copy_from_device(buf.ctypes.data, imports[(k, j, 7)], 4096) == 0
+                    assert (buf == 0xC0 + j).all()
+        for (k, j, i), va in imports.items():
+            lib.amem_del_alloc_info(va, 0, 0)
+            lib.amem_vmm_free(va, int(owned[j].alloc[i]), 0)
+        for r in owned:
+            r.free()
     finally:
         lib.amem_mem_resume(0, 0)
         lib.amem_ipc_act_as(-1)

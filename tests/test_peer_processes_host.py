@@ -38,6 +38,15 @@ def test_processes_through_pause_and_resume(standin, world):
     run_world(world, lib_path=standin, gid_base=0x6800)
 
 
+def test_four_processes_at_the_full_shape_of_configuration_5(standin):
+    """Benchmark configuration 5 at its stated shape between real processes: 4 processes, each owning all
+    256 regions of configuration 2's layout (1,216 MiB, seeds 4-7), exporting 256 descriptors to each of
+    the three others and importing their 768. Per resume every process re-exports 768 descriptors over
+    three sockets and its service thread maps 768 received ones (amem_nccl.cpp:517-526, :633-662); the
+    descriptor count of every process is the same after each cycle as before the first."""
+    run_world(4, lib_path=standin, gid_base=0x6c00, nreg=256, phase_timeout=300)
+
+
 def _owner_that_dies(ipc_dir, gid, lib_path, conn, ctrl):
     os.environ.update(AMEM_ENABLE="1", GMM_LOG="1", GMM_IPC_DIR=ipc_dir, AMEM_GROUPID=str(gid), AMEM_SLOT="0")
     from asystem_amem_amd import binding as B, harness as H
