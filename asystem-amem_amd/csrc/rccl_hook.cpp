@@ -38,17 +38,34 @@
 //                                  for layouts in which RCCL does not hand these buffers to another process
 //                                  over legacy IPC (one rank per node, or P2P over IPC disabled).
 //
+//   hipIpcGetMemHandle             a mapping served in place of a plain allocation cannot be shared that way:
+//                                  for such an address the call is refused and one ERROR line says why and
+//                                  what to set (NCCL_P2P_DISABLE=1, or no AMEM_HOOK_PLAIN_ALLOC); every other
+//                                  address is forwarded
+//
+// amem_rccl_hook_exclude(ptr) takes one buffer back out of the registry by hand: the manual form of the
+// reference's removals before NIC registration, for callers that know which buffers they register.
+// amem_rccl_hook_unserved_bytes() and a line at process exit say how much RCCL allocated that the hook left
+// alone (below the threshold; uncached, fine-grained or otherwise flagged; not servable).
+//
 // Calls made by anything else (the pause/resume engine itself, the application) pass through
 // untouched. The module a call comes from is found from its return address.
+//
+// Locking: g_mtx guards this file's maps and nothing else. No call into the HIP runtime or into
+// libamem_nccl is made while it is held (the engine calls hipFree, which lands here, while it holds
+// its own locks; a hook that called into the engine under g_mtx would close a cycle).
 #define _GNU_SOURCE 1
 #include <dlfcn.h>
+#include <errno.h>
 #include <fcntl.h>
+#include <signal.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <atomic>
 #include <string>
 
 #include <mutex>
@@ -68,17 +85,23 @@ struct Pending {
   uint64_t handle;
 };
 
+// The maps below are never destroyed: hipFree and the other hooks may still be called by other
+// libraries' clean-up code after this library's static objects would have been torn down.
 std::mutex g_mtx;
-std::unordered_map<uint64_t, Pending> g_mapped;      // RCCL mappings seen at hipMemMap
-std::unordered_set<uint64_t> g_registered;           // those handed to the registry
+std::unordered_map<uint64_t, Pending>& g_mapped = *new std::unordered_map<uint64_t, Pending>();      // RCCL mappings seen at hipMemMap
+std::unordered_set<uint64_t>& g_registered = *new std::unordered_set<uint64_t>();           // those handed to the registry
 struct Owner {
   int slot;         // slot of the owning process, -1 when unknown
-  uint64_t handle;  // the owner's handle value
+  uint64_t handle;  // the owner's handle value when the descriptor was exported (it changes with every resume)
+  uint64_t va;      // the owner's address of the region (it never changes); 0 when unknown
+  // What the importer names the region by when it registers with the owner: the address where it is
+  // known, because a handle value noted at export time is dead after the owner's next resume.
+  uint64_t name() const { return va ? va : handle; }
 };
-std::unordered_map<uint64_t, Owner> g_imported_handles;   // handles RCCL imported from a peer -> who owns the memory
-std::unordered_map<std::string, Owner> g_exports;         // descriptor identity -> this process's handle behind it
-std::unordered_map<uint64_t, std::string> g_export_of;    // exported handle -> descriptor identity (to forget it again)
-std::unordered_map<uint64_t, std::string> g_export_at;    // address the exported handle was mapped at -> identity; the
+std::unordered_map<uint64_t, Owner>& g_imported_handles = *new std::unordered_map<uint64_t, Owner>();   // handles RCCL imported from a peer -> who owns the memory
+std::unordered_map<std::string, Owner>& g_exports = *new std::unordered_map<std::string, Owner>();         // descriptor identity -> this process's handle behind it
+std::unordered_map<uint64_t, std::string>& g_export_of = *new std::unordered_map<uint64_t, std::string>();    // exported handle -> descriptor identity (to forget it again)
+std::unordered_map<uint64_t, std::string>& g_export_at = *new std::unordered_map<uint64_t, std::string>();    // address the exported handle was mapped at -> identity; the
                                                           // handle value changes with every resume, the address never
 int g_verbose = -1;
 
@@ -156,7 +179,7 @@ HOOK_API hipError_t hipMemSetAccess(void* ptr, size_t size, const hipMemAccessDe
   hipError_t e = fn(ptr, size, desc, count);
   if (e != hipSuccess || !from_rccl(__builtin_return_address(0))) return e;
   Pending p = {0, 0};
-  Owner owner = {-1, 0};
+  Owner owner = {-1, 0, 0};
   bool fresh = false, imported = false;
   {
     std::lock_guard<std::mutex> lk(g_mtx);
@@ -179,7 +202,7 @@ HOOK_API hipError_t hipMemSetAccess(void* ptr, size_t size, const hipMemAccessDe
     if (imported)
       // the shape of the reference's hook in ncclP2pImportShareableBuffer (nccl_patch/nccl_2.27.5-1.diff:572-579)
       rc = amem_add_alloc_info((uint64_t)(uintptr_t)ptr, p.size, AMEM_TYPE_PEER_POSIX, dev, p.handle, owner.slot,
-                               owner.handle, NULL, AMEM_CALLER_P2P_PEER);
+                               owner.name(), NULL, AMEM_CALLER_P2P_PEER);
     else
       // the shape of the reference's hook in ncclCuMemAlloc (nccl_patch/nccl_2.27.5-1.diff:278-280)
       rc = amem_add_alloc_info((uint64_t)(uintptr_t)ptr, p.size, AMEM_TYPE_LOCAL, dev, p.handle, -1, 0, NULL,
@@ -225,7 +248,7 @@ HOOK_API hipError_t hipMemImportFromShareableHandle(hipMemGenericAllocationHandl
       "hipMemImportFromShareableHandle");
   hipError_t e = fn(handle, osHandle, shHandleType);
   if (e == hipSuccess && handle && from_rccl(__builtin_return_address(0))) {
-    Owner owner = {-1, 0};
+    Owner owner = {-1, 0, 0};
     if (shHandleType == hipMemHandleTypePosixFileDescriptor) {
       const std::string id = identity_of((int)(uintptr_t)osHandle);
       bool found = false;
@@ -240,14 +263,29 @@ HOOK_API hipError_t hipMemImportFromShareableHandle(hipMemGenericAllocationHandl
       if (!found && !id.empty()) {
         // exported by another process: it left a note under the descriptor's identity
         // (only a note this user wrote counts, and a symbolic link in its place is not followed)
-        const int nfd = open(export_file(id).c_str(), O_RDONLY | O_NOFOLLOW | O_CLOEXEC);
+        const std::string path = export_file(id);
+        const int nfd = open(path.c_str(), O_RDONLY | O_NOFOLLOW | O_CLOEXEC);
         struct stat st;
         if (nfd >= 0 && fstat(nfd, &st) == 0 && S_ISREG(st.st_mode) && st.st_uid == geteuid()) {
-          char buf[96] = {0};
+          char buf[128] = {0};
           const ssize_t n = read(nfd, buf, sizeof(buf) - 1);
-          int slot = -1;
-          unsigned long long h = 0;
-          if (n > 0 && sscanf(buf, "%d %llx", &slot, &h) == 2 && slot >= 0 && slot < AMEM_MAX_DEVS) owner = {slot, (uint64_t)h};
+          int slot = -1, pid = 0;
+          unsigned long long h = 0, va = 0;
+          const int fields = n > 0 ? sscanf(buf, "%d %llx %d %llx", &slot, &h, &pid, &va) : 0;
+          if (fields >= 3 && slot >= 0 && slot < AMEM_MAX_DEVS) {
+            // Identities are reused (the inode number of a descriptor's file is), so a note may be what a
+            // process that has died left behind. It counts only while its writer is alive and somebody
+            // holds the slot it names; a stale one is removed.
+            const bool writer_alive = pid > 0 && (kill((pid_t)pid, 0) == 0 || errno == EPERM);
+            if (writer_alive && amem_ipc_peer_alive(slot)) {
+              owner = {slot, (uint64_t)h, fields >= 4 ? (uint64_t)va : 0};
+            } else {
+              if (verbose()) fprintf(stderr, "AMEM [DEBG] rccl_hook: note %s is stale (pid %d %s, slot %d %s); ignored\n",
+                                     path.c_str(), pid, writer_alive ? "alive" : "gone", slot,
+                                     amem_ipc_peer_alive(slot) ? "held" : "free");
+              unlink(path.c_str());
+            }
+          }
         }
         if (nfd >= 0) close(nfd);
       }
@@ -271,16 +309,18 @@ HOOK_API hipError_t hipMemExportToShareableHandle(void* shareableHandle, hipMemG
     const int slot = amem_get_slot();
     if (!id.empty() && slot >= 0) {
       const uint64_t h = (uint64_t)(uintptr_t)handle;
+      // (asked before the lock is taken: the look-up takes the registry's locks)
+      int dev = 0;
+      (void)hipGetDevice(&dev);
+      const uint64_t va = amem_handle_lookup(dev, h);
       std::string stale;
       {
         std::lock_guard<std::mutex> lk(g_mtx);
         auto old = g_export_of.find(h);
         if (old != g_export_of.end() && old->second != id) stale = old->second;
-        g_exports[id] = {slot, h};
+        g_exports[id] = {slot, h, va};
         g_export_of[h] = id;
-        int dev = 0;
-        (void)hipGetDevice(&dev);
-        if (uint64_t va = amem_handle_lookup(dev, h)) g_export_at[va] = id;
+        if (va) g_export_at[va] = id;
       }
       if (!stale.empty()) unlink(export_file(stale).c_str());
       // the note is this user's alone, and is never written through a link somebody else left under its name
@@ -288,8 +328,9 @@ HOOK_API hipError_t hipMemExportToShareableHandle(void* shareableHandle, hipMemG
       unlink(note.c_str());
       const int nfd = open(note.c_str(), O_WRONLY | O_CREAT | O_EXCL | O_NOFOLLOW | O_CLOEXEC, 0600);
       if (nfd >= 0) {
-        char buf[96];
-        const int n = snprintf(buf, sizeof(buf), "%d %llx %d\n", slot, (unsigned long long)h, (int)getpid());
+        char buf[128];
+        const int n = snprintf(buf, sizeof(buf), "%d %llx %d %llx\n", slot, (unsigned long long)h, (int)getpid(),
+                               (unsigned long long)va);
         if (write(nfd, buf, (size_t)n) != n && verbose()) fprintf(stderr, "AMEM [WARN] rccl_hook: short write to %s\n", note.c_str());
         close(nfd);
       }
@@ -319,7 +360,17 @@ HOOK_API hipError_t hipMemRelease(hipMemGenericAllocationHandle_t handle) {
 // ---- plain allocations served through the virtual-memory API (opt-in) ----
 
 namespace {
-std::unordered_map<uint64_t, uint64_t> g_substituted;  // address handed to RCCL -> mapped size
+std::unordered_map<uint64_t, uint64_t>& g_substituted = *new std::unordered_map<uint64_t, uint64_t>();  // address handed to RCCL -> mapped size
+// RCCL's plain allocations that were left as they are, by reason (only kept while the opt-in mode is on)
+enum LeftWhy { LEFT_SMALL = 0, LEFT_FLAGGED = 1, LEFT_UNSERVABLE = 2, LEFT_KINDS = 3 };
+struct Left { uint64_t size; int why; };
+std::unordered_map<uint64_t, Left>& g_left = *new std::unordered_map<uint64_t, Left>();
+uint64_t g_left_bytes[LEFT_KINDS] = {0, 0, 0};        // held by RCCL right now
+uint64_t g_left_total[LEFT_KINDS] = {0, 0, 0};        // allocated since load, for the line at exit
+uint64_t g_served_total = 0, g_served_count = 0;        // since load, for the line at exit
+// Entries in g_substituted plus g_left. hipFree is called by everybody, the engine included; while
+// this is zero it goes straight through without touching g_mtx.
+std::atomic<long> g_tracked{0};
 long long g_plain_min = -2;
 size_t plain_alloc_min() {
   if (g_plain_min == -2) {
@@ -327,6 +378,20 @@ size_t plain_alloc_min() {
     g_plain_min = (e && atoll(e) > 0) ? atoll(e) : 0;
   }
   return (size_t)g_plain_min;
+}
+
+void note_left(void* ptr, size_t size, int why) {
+  if (!ptr) return;
+  std::lock_guard<std::mutex> lk(g_mtx);
+  auto ins = g_left.emplace((uint64_t)(uintptr_t)ptr, Left{(uint64_t)size, why});
+  if (ins.second) { g_left_bytes[why] += size; g_left_total[why] += size; g_tracked.fetch_add(1, std::memory_order_relaxed); }
+}
+
+// The served mapping that holds `addr`, or 0. (g_mtx held by the caller.)
+uint64_t served_base_of(uint64_t addr) {
+  for (auto& kv : g_substituted)
+    if (addr >= kv.first && addr < kv.first + kv.second) return kv.first;
+  return 0;
 }
 }  // namespace
 
@@ -342,6 +407,9 @@ static bool serve_plain(void** ptr, size_t size) {
   {
     std::lock_guard<std::mutex> lk(g_mtx);
     g_substituted[va] = asz;
+    g_tracked.fetch_add(1, std::memory_order_relaxed);
+    g_served_total += asz;
+    g_served_count++;
     if (rc == 0) g_registered.insert(va);
   }
   if (verbose()) fprintf(stderr, "AMEM [DEBG] rccl_hook: plain allocation of %zu bytes served as a mapping at %llx of %llu bytes, registered rc %d\n",
@@ -353,21 +421,33 @@ static bool serve_plain(void** ptr, size_t size) {
 HOOK_API hipError_t hipMalloc(void** ptr, size_t size) {
   static auto fn = real<hipError_t (*)(void**, size_t)>("hipMalloc");
   const size_t min = plain_alloc_min();
-  if (min && ptr && size >= min && from_rccl(__builtin_return_address(0)) && serve_plain(ptr, size)) return hipSuccess;
-  return fn(ptr, size);
+  const bool rccl = min && ptr && from_rccl(__builtin_return_address(0));
+  if (rccl && size >= min && serve_plain(ptr, size)) return hipSuccess;
+  hipError_t e = fn(ptr, size);
+  if (rccl && e == hipSuccess) note_left(*ptr, size, size >= min ? LEFT_UNSERVABLE : LEFT_SMALL);
+  return e;
 }
 
 HOOK_API hipError_t hipFree(void* ptr) {
   static auto fn = real<hipError_t (*)(void*)>("hipFree");
+  if (!ptr || g_tracked.load(std::memory_order_relaxed) == 0) return fn(ptr);
   uint64_t asz = 0;
   bool was_registered = false;
-  if (ptr) {
+  {
     std::lock_guard<std::mutex> lk(g_mtx);
     auto it = g_substituted.find((uint64_t)(uintptr_t)ptr);
     if (it != g_substituted.end()) {
       asz = it->second;
       g_substituted.erase(it);
+      g_tracked.fetch_sub(1, std::memory_order_relaxed);
       was_registered = g_registered.erase((uint64_t)(uintptr_t)ptr) > 0;
+    } else {
+      auto lf = g_left.find((uint64_t)(uintptr_t)ptr);
+      if (lf != g_left.end()) {
+        g_left_bytes[lf->second.why] -= lf->second.size;
+        g_left.erase(lf);
+        g_tracked.fetch_sub(1, std::memory_order_relaxed);
+      }
     }
   }
   if (!asz) return fn(ptr);
@@ -384,11 +464,33 @@ HOOK_API hipError_t hipExtMallocWithFlags(void** ptr, size_t size, unsigned int 
   // flags 0 is an ordinary allocation under another name (this is how RCCL 2.27 allocates everything);
   // fine-grained, uncached and signal memory keep their own semantics and are never served differently
   const size_t min = plain_alloc_min();
-  const bool rccl = (min || verbose()) && from_rccl(__builtin_return_address(0));
-  if (rccl && min && ptr && flags == hipDeviceMallocDefault && size >= min && serve_plain(ptr, size)) return hipSuccess;
+  const bool rccl = (min || verbose()) && ptr && from_rccl(__builtin_return_address(0));
+  if (rccl && min && flags == hipDeviceMallocDefault && size >= min && serve_plain(ptr, size)) return hipSuccess;
   if (rccl && verbose() && size >= (1u << 20))
     fprintf(stderr, "AMEM [DEBG] rccl_hook: hipExtMallocWithFlags(%zu, flags %x) left as it is\n", size, flags);
-  return fn(ptr, size, flags);
+  hipError_t e = fn(ptr, size, flags);
+  if (rccl && min && e == hipSuccess)
+    note_left(*ptr, size, flags != hipDeviceMallocDefault ? LEFT_FLAGGED : size >= min ? LEFT_UNSERVABLE : LEFT_SMALL);
+  return e;
+}
+
+// A mapping served in place of a plain allocation cannot become a legacy IPC handle, which is how a
+// multi-rank RCCL shares its buffers between the processes of one node unless told otherwise. For such
+// an address the call is refused here (what the runtime does with a virtual-memory mapping handed to
+// this call is not relied upon) and one line says why; every other address goes through untouched.
+HOOK_API hipError_t hipIpcGetMemHandle(hipIpcMemHandle_t* handle, void* devPtr) {
+  static auto fn = real<hipError_t (*)(hipIpcMemHandle_t*, void*)>("hipIpcGetMemHandle");
+  uint64_t base = 0;
+  if (devPtr && g_tracked.load(std::memory_order_relaxed) != 0) {
+    std::lock_guard<std::mutex> lk(g_mtx);
+    base = served_base_of((uint64_t)(uintptr_t)devPtr);
+  }
+  if (!base) return fn(handle, devPtr);
+  fprintf(stderr, "AMEM [ERRO] rccl_hook: hipIpcGetMemHandle(%p) refused: the buffer at %llx is a virtual-memory mapping the hook "
+          "served in place of a plain allocation (AMEM_HOOK_PLAIN_ALLOC), and such a mapping cannot be shared over legacy IPC. "
+          "Run RCCL with NCCL_P2P_DISABLE=1 (or one rank per node), or unset AMEM_HOOK_PLAIN_ALLOC.\n",
+          devPtr, (unsigned long long)base);
+  return hipErrorInvalidValue;
 }
 
 // Bytes currently served to RCCL through the virtual-memory API in place of plain allocations.
@@ -399,8 +501,65 @@ HOOK_API uint64_t amem_rccl_hook_served_bytes(void) {
   return n;
 }
 
+// Bytes RCCL currently holds in plain allocations that the hook left alone while AMEM_HOOK_PLAIN_ALLOC is
+// set: `below_threshold` were smaller than the variable's value, `flagged` asked for uncached, fine-grained
+// or otherwise special memory (which keeps its semantics), `unservable` could not be created through the
+// virtual-memory API. Any pointer may be NULL. Returns the sum.
+HOOK_API uint64_t amem_rccl_hook_unserved_bytes(uint64_t* below_threshold, uint64_t* flagged, uint64_t* unservable) {
+  std::lock_guard<std::mutex> lk(g_mtx);
+  if (below_threshold) *below_threshold = g_left_bytes[LEFT_SMALL];
+  if (flagged) *flagged = g_left_bytes[LEFT_FLAGGED];
+  if (unservable) *unservable = g_left_bytes[LEFT_UNSERVABLE];
+  return g_left_bytes[LEFT_SMALL] + g_left_bytes[LEFT_FLAGGED] + g_left_bytes[LEFT_UNSERVABLE];
+}
+
 // Number of RCCL mappings currently mirrored into the registry (for tests and diagnostics).
 HOOK_API int64_t amem_rccl_hook_registered(void) {
   std::lock_guard<std::mutex> lk(g_mtx);
   return (int64_t)g_registered.size();
+}
+
+// Take the buffer that holds `ptr` out of the registry: a pause no longer releases it and it keeps its
+// memory. The manual form of what the reference does just before a buffer is registered with a NIC
+// (nccl_patch/nccl_2.27.5-1.diff:309-312, :364-367), for callers that know which buffers they register;
+// the hook cannot see those sites itself. 0 done; 1 the address belongs to nothing the hook registered;
+// 2 refused while paused (the buffer's memory is already gone and only the registry can bring it back).
+HOOK_API int amem_rccl_hook_exclude(void* ptr) {
+  if (!ptr) return 1;
+  if (amem_check_paused(0)) return 2;
+  const uint64_t addr = (uint64_t)(uintptr_t)ptr;
+  uint64_t base = 0;
+  {
+    std::lock_guard<std::mutex> lk(g_mtx);
+    for (uint64_t va : g_registered) {
+      uint64_t size = 0;
+      auto m = g_mapped.find(va);
+      if (m != g_mapped.end()) size = m->second.size;
+      auto sub = g_substituted.find(va);
+      if (sub != g_substituted.end()) size = sub->second;
+      if (addr >= va && addr < va + (size ? size : 1)) { base = va; break; }
+    }
+    if (base) g_registered.erase(base);
+  }
+  if (!base) return 1;
+  (void)amem_del_alloc_info(base, 0, 0);
+  if (verbose()) fprintf(stderr, "AMEM [DEBG] rccl_hook: %llx taken out of the registry on request\n", (unsigned long long)base);
+  return 0;
+}
+
+// What the opt-in mode did for this process, once, when it ends: how much of what RCCL allocated could be
+// put into the registry, and how much could not and why.
+static void __attribute__((destructor)) amem_rccl_hook_summary(void) {
+  if (plain_alloc_min() == 0) return;
+  uint64_t total, count, left[LEFT_KINDS];
+  {
+    std::lock_guard<std::mutex> lk(g_mtx);
+    total = g_served_total; count = g_served_count;
+    for (int k = 0; k < LEFT_KINDS; ++k) left[k] = g_left_total[k];
+  }
+  fprintf(stderr, "AMEM [INFO] rccl_hook: AMEM_HOOK_PLAIN_ALLOC=%zu, RCCL's plain allocations since load: %.1f MiB in %llu "
+          "allocations served through the virtual-memory API and registered; %.1f MiB left alone (%.1f MiB below the "
+          "threshold, %.1f MiB uncached / fine-grained, %.1f MiB not servable)\n", plain_alloc_min(), total / 1048576.0,
+          (unsigned long long)count, (left[0] + left[1] + left[2]) / 1048576.0, left[LEFT_SMALL] / 1048576.0,
+          left[LEFT_FLAGGED] / 1048576.0, left[LEFT_UNSERVABLE] / 1048576.0);
 }

@@ -149,6 +149,17 @@ hipError_t hipFree(void* p) {
   free(p);
   return hipSuccess;
 }
+hipError_t hipExtMallocWithFlags(void** p, size_t n, unsigned int) { return hipMalloc(p, n); }
+hipError_t hipIpcGetMemHandle(hipIpcMemHandle_t* h, void* p) {
+  std::lock_guard<std::mutex> lk(g_mtx);
+  if (!h || g_blocks.find((uintptr_t)p) == g_blocks.end()) return fail(hipErrorInvalidValue);
+  memset(h, 0, sizeof(*h));
+  return hipSuccess;
+}
+hipError_t hipMemGetAllocationGranularity(size_t* g, const hipMemAllocationProp*, hipMemAllocationGranularity_flags) {
+  *g = 4096;
+  return hipSuccess;
+}
 hipError_t hipHostMalloc(void** p, size_t n, unsigned int) { return block_alloc(p, n, false); }
 hipError_t hipHostFree(void* p) { return hipFree(p); }
 hipError_t hipHostGetDevicePointer(void** dp, void* hp, unsigned int) { *dp = hp; return hipSuccess; }

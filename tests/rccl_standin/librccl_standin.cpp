@@ -72,3 +72,25 @@ extern "C" __attribute__((visibility("default"))) int standin_import_map(int fd,
   if (hipMemSetAccess(*ptr, size, &acc, 1) != hipSuccess) return 5;
   return 0;
 }
+
+// RCCL 2.27 keeps its own buffers in plain allocations (hipExtMallocWithFlags with flags 0, fine-grained
+// memory for what the host polls). These three make the same calls from a file named librccl_*.so.
+// (Each call is followed by more code on purpose: the hook tells RCCL's calls by their return address,
+// and a call compiled into a jump would return straight into this function's caller.)
+extern "C" __attribute__((visibility("default"))) int standin_plain_alloc(void** ptr, size_t size, unsigned int flags, int use_ext) {
+  const hipError_t e = use_ext ? hipExtMallocWithFlags(ptr, size, flags) : hipMalloc(ptr, size);
+  if (e != hipSuccess) (void)hipGetLastError();
+  return (int)e;
+}
+extern "C" __attribute__((visibility("default"))) int standin_plain_free(void* ptr) {
+  const hipError_t e = hipFree(ptr);
+  if (e != hipSuccess) (void)hipGetLastError();
+  return (int)e;
+}
+// What a multi-rank RCCL does with a buffer it wants a neighbour process to reach over legacy IPC.
+extern "C" __attribute__((visibility("default"))) int standin_ipc_handle(void* ptr) {
+  hipIpcMemHandle_t h;
+  hipError_t e = hipIpcGetMemHandle(&h, ptr);
+  (void)hipGetLastError();
+  return (int)e;
+}

@@ -213,7 +213,7 @@ tab = H.region_table(lib, 0)
 assert len(tab) == 6 and hook.amem_rccl_hook_registered() == 6
 for (p, n, _), q in zip(owned, imports):
     assert tab[q]["type"] == B.TYPE_PEER_POSIX and tab[q]["alloc_sz"] == n and tab[q]["tags"] == B.CALLER_P2P_PEER
-    assert tab[q]["mc_handle"] == tab[p]["handle"]                 # the owner's handle value travelled with the descriptor
+    assert tab[q]["mc_handle"] == p                                # the importer names the region by the owner's address, which no resume changes
     assert tab[p]["has_peer"] == 1 and tab[p]["peers"][slot_b] == q
 lib.ncclPause(None); lib.ncclResume(None)                          # warm cycle
 free0 = H.mem_free(lib)
@@ -287,7 +287,13 @@ uid, comm = UID(), C.c_void_p()
 assert rccl.ncclGetUniqueId(C.byref(uid)) == 0
 assert rccl.ncclCommInitRank(C.byref(comm), 1, uid, 0) == 0
 served, regions = hook.amem_rccl_hook_served_bytes(), hook.amem_rccl_hook_registered()
-print("served to RCCL through the virtual-memory API: %.1f MiB in %d regions" % (served / 2**20, regions))
+hook.amem_rccl_hook_unserved_bytes.restype = C.c_uint64
+hook.amem_rccl_hook_unserved_bytes.argtypes = [C.POINTER(C.c_uint64)] * 3
+small, flagged, unservable = C.c_uint64(), C.c_uint64(), C.c_uint64()
+left = hook.amem_rccl_hook_unserved_bytes(C.byref(small), C.byref(flagged), C.byref(unservable))
+print("one-rank communicator of the real RCCL: %.1f MiB in %d regions served through the virtual-memory API; left alone %.1f MiB "
+      "(%.1f below the 1 MiB threshold, %.1f uncached / fine-grained, %.1f not servable)" %
+      (served / 2**20, regions, left / 2**20, small.value / 2**20, flagged.value / 2**20, unservable.value / 2**20))
 if served == 0:
     print("this RCCL made no plain allocation of 1 MiB or more"); print("rccl skipped"); sys.exit(0)
 assert lib.amem_region_count(0) == regions
@@ -331,7 +337,7 @@ print("rccl plain ok")
 '''
 
 
-def test_real_rccl_buffers_served_through_the_vmm_api_are_released_and_restored(gpu):
+def test_real_rccl_buffers_served_through_the_vmm_api_are_released_and_restored(gpu, measured):
     """A real communicator's own memory in the registry (what the reference's hooks in ncclCuMemAlloc are
     for, nccl_patch/nccl_2.27.5-1.diff:278-280). The RCCL of this ROCm release keeps its buffers in plain
     allocations, which nothing can unmap; with AMEM_HOOK_PLAIN_ALLOC set, the hook serves RCCL's plain
@@ -343,5 +349,110 @@ def test_real_rccl_buffers_served_through_the_vmm_api_are_released_and_restored(
     r = subprocess.run([sys.executable, "-c", PLAIN_ALLOC_CHILD, ROOT], env=env, capture_output=True, text=True, timeout=240)
     assert r.returncode == 0 and ("rccl plain ok" in r.stdout or "rccl skipped" in r.stdout), \
         (r.returncode, r.stdout[-3000:], r.stderr[-3000:])
+    for line in r.stdout.splitlines():
+        if line.startswith("one-rank communicator") or line.startswith("released per pause"):
+            measured(line)
     if "rccl skipped" in r.stdout:
         pytest.skip("librccl.so is not loadable here, or it made no plain allocation the hook serves")
+
+
+GUARDS_CHILD = r'''
+import ctypes as C, os, sys
+import numpy as np
+root, standin = sys.argv[1], sys.argv[2]
+sys.path.insert(0, root)
+libdir = os.path.join(root, "asystem-amem_amd", "lib")
+hook = C.CDLL(os.path.join(libdir, "libamem_rccl_hook.so"), mode=C.RTLD_GLOBAL)
+from asystem_amem_amd import binding as B, harness as H
+lib = B.load()
+rccl = C.CDLL(standin, mode=C.RTLD_GLOBAL)
+rccl.standin_plain_alloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t, C.c_uint, C.c_int]
+rccl.standin_plain_free.argtypes = [C.c_void_p]
+rccl.standin_ipc_handle.argtypes = [C.c_void_p]
+hook.amem_rccl_hook_registered.restype = C.c_int64
+hook.amem_rccl_hook_served_bytes.restype = C.c_uint64
+hook.amem_rccl_hook_unserved_bytes.restype = C.c_uint64
+hook.amem_rccl_hook_unserved_bytes.argtypes = [C.POINTER(C.c_uint64)] * 3
+hook.amem_rccl_hook_exclude.argtypes = [C.c_void_p]
+MiB = 1 << 20
+FINE_GRAINED = 1                                                   # hipDeviceMallocFinegrained
+rng = np.random.default_rng(51)
+
+def unserved():
+    a, b, c = C.c_uint64(), C.c_uint64(), C.c_uint64()
+    total = hook.amem_rccl_hook_unserved_bytes(C.byref(a), C.byref(b), C.byref(c))
+    assert total == a.value + b.value + c.value
+    return a.value, b.value, c.value
+
+# what the threshold of 1 MiB does with five allocations made the way RCCL makes them
+big, big2, small, fine, plain = [C.c_void_p() for _ in range(5)]
+assert rccl.standin_plain_alloc(C.byref(big), 8 * MiB, 0, 1) == 0      # served and registered
+assert rccl.standin_plain_alloc(C.byref(big2), 4 * MiB, 0, 0) == 0     # served and registered (hipMalloc)
+assert rccl.standin_plain_alloc(C.byref(small), 256 << 10, 0, 1) == 0  # below the threshold
+assert rccl.standin_plain_alloc(C.byref(fine), 2 * MiB, FINE_GRAINED, 1) == 0   # keeps its semantics
+assert hook.amem_rccl_hook_served_bytes() == 12 * MiB and hook.amem_rccl_hook_registered() == 2
+assert unserved() == (256 << 10, 2 * MiB, 0)
+assert lib.amem_region_count(0) == 2
+data = {}
+for p, n in ((big, 8 * MiB), (big2, 4 * MiB)):
+    d = rng.integers(1, 256, n, dtype=np.uint8)
+    assert lib.amem_copy_to_device(p.value, d.ctypes.data, n) == 0
+    data[p.value] = d
+
+# (a) legacy IPC: refused for a served mapping with a line that says what to do, untouched for the rest
+assert rccl.standin_ipc_handle(big.value) != 0
+assert rccl.standin_ipc_handle(big.value + 4096) != 0              # any address inside it
+assert rccl.standin_ipc_handle(small.value) == 0                   # an ordinary allocation still gets its handle
+sys.stderr.flush()
+
+# (c) a buffer the caller registers with a NIC is taken out of the registry by hand
+lib.ncclPause(None); lib.ncclResume(None)                          # warm cycle
+free0 = H.mem_free(lib)
+assert lib.ncclPause(None) == 0
+assert H.mem_free(lib) - free0 >= 12 * MiB - 2 * MiB              # both served buffers are released
+assert hook.amem_rccl_hook_exclude(big2.value) == 2                # not while paused: its memory is gone
+assert lib.ncclResume(None) == 0
+assert hook.amem_rccl_hook_exclude(big2.value + 8192) == 0         # by any address inside the buffer
+assert hook.amem_rccl_hook_exclude(big2.value) == 1                # it is no longer the hook's
+assert hook.amem_rccl_hook_exclude(small.value) == 1               # never was
+assert lib.amem_region_count(0) == 1 and hook.amem_rccl_hook_registered() == 1
+assert hook.amem_rccl_hook_served_bytes() == 12 * MiB              # still a mapping the hook has to free one day
+free1 = H.mem_free(lib)
+assert lib.ncclPause(None) == 0
+released = H.mem_free(lib) - free1
+assert 8 * MiB - 2 * MiB <= released < 12 * MiB - MiB, released    # only the buffer still registered went
+out = np.empty(4 * MiB, dtype=np.uint8)                            # the excluded one is readable while paused
+assert lib.amem_copy_from_device(out.ctypes.data, big2.value, out.nbytes) == 0 and np.array_equal(out, data[big2.value])
+assert lib.ncclResume(None) == 0
+for p, d in data.items():
+    out = np.empty(d.nbytes, dtype=np.uint8)
+    assert lib.amem_copy_from_device(out.ctypes.data, p, d.nbytes) == 0 and np.array_equal(out, d)
+for p in (big, big2, small, fine):
+    assert rccl.standin_plain_free(p.value) == 0
+assert hook.amem_rccl_hook_served_bytes() == 0 and hook.amem_rccl_hook_registered() == 0 and unserved() == (0, 0, 0)
+assert lib.amem_region_count(0) == 0 and lib.amem_handle_count(0) == 0
+print("rccl hook guards ok")
+'''
+
+
+def test_hook_guards_for_served_allocations(gpu, tmp_path):
+    """The opt-in mode's guard rails, with a caller that allocates the way RCCL 2.27 does (a file named
+    librccl_*.so calling hipExtMallocWithFlags / hipMalloc): what is served and what is left alone is
+    counted by reason; hipIpcGetMemHandle on a served mapping fails with one line that names
+    AMEM_HOOK_PLAIN_ALLOC and NCCL_P2P_DISABLE=1, and works as ever for ordinary memory; a buffer taken
+    out by amem_rccl_hook_exclude (the manual form of the reference's removal before NIC registration,
+    nccl_patch/nccl_2.27.5-1.diff:309-312, :364-367) keeps its memory through a pause; the line at exit
+    says how much could be registered and how much not."""
+    standin = str(tmp_path / "librccl_standin.so")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    subprocess.run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-D__HIP_PLATFORM_AMD__",
+                    "-I" + os.path.join(rocm, "include"), os.path.join(ROOT, "tests", "rccl_standin", "librccl_standin.cpp"),
+                    "-o", standin, "-L" + os.path.join(rocm, "lib"), "-lamdhip64"], check=True, capture_output=True, text=True)
+    env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="1", AMEM_IPC="0", AMEM_HOOK_PLAIN_ALLOC=str(1 << 20))
+    r = subprocess.run([sys.executable, "-c", GUARDS_CHILD, ROOT, standin], env=env, capture_output=True, text=True, timeout=240)
+    assert r.returncode == 0 and "rccl hook guards ok" in r.stdout, (r.returncode, r.stdout[-3000:], r.stderr[-3000:])
+    errs = [l for l in r.stderr.splitlines() if "hipIpcGetMemHandle" in l and "[ERRO]" in l]
+    assert len(errs) == 2 and all("AMEM_HOOK_PLAIN_ALLOC" in l and "NCCL_P2P_DISABLE=1" in l for l in errs), r.stderr[-3000:]
+    summary = [l for l in r.stderr.splitlines() if "RCCL's plain allocations since load" in l]
+    assert len(summary) == 1 and "12.0 MiB in 2 allocations served" in summary[0], r.stderr[-3000:]
+    assert "2.2 MiB left alone (0.2 MiB below the threshold, 2.0 MiB uncached / fine-grained, 0.0 MiB not servable)" in summary[0], summary
