@@ -57,7 +57,7 @@ class CycleStats(C.Structure):
         "k1_launches", "k2_launches", "k3_launches", "footprint_bytes", "parked_bytes", "zero_chunks",
         "total_chunks", "local_regions", "peer_regions", "dma_bytes", "kernel_bytes", "slab_bytes",
         "verify_mismatch")] + [(n, C.c_double) for n in (
-        "pause_pool_ms", "pause_scratch_ms", "pause_sync_ms", "resume_scratch_ms")] + [("resume_dma_bytes", C.c_uint64)]
+        "pause_pool_ms", "pause_scratch_ms", "pause_sync_ms", "resume_scratch_ms")] + [("resume_dma_bytes", C.c_uint64), ("pause_narrow_launches", C.c_uint64)]
 
     def as_dict(self):
         return {k: getattr(self, k) for k, _ in self._fields_}
@@ -126,12 +126,18 @@ _SIGNATURES = {
                                    C.POINTER(C.c_float)]),
     "amem_scatter_unpack": (C.c_int, [C.POINTER(CopyDesc), C.c_uint64, C.c_void_p, C.c_uint64, C.c_int,
                                       C.POINTER(C.c_float)]),
+}
+
+# include/amem_testing.h: measurement and test helpers, same library
+_TESTING_SIGNATURES = {
     "amem_probe_link": (C.c_int, [C.c_uint64, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "amem_probe_unmap": (C.c_int, [C.c_int, C.c_uint64, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_double)]),
     "amem_calib_copy": (C.c_int, [C.c_uint64, C.c_int, C.POINTER(C.c_float)]),
     "amem_copy_to_device": (C.c_int, [C.c_uint64, C.c_void_p, C.c_uint64]),
     "amem_copy_from_device": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64]),
     "amem_device_mem_info": (C.c_int, [C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "amem_device_count": (C.c_int, []),
+    "amem_device_pci_bus_id": (C.c_int, [C.c_char_p, C.c_int]),
 }
 
 # The reference's own C++-linkage names, as its library exports them.
@@ -146,7 +152,7 @@ _lib = None
 
 
 def load(path=None):
-    """Load the library (once) and declare every entry point of include/amem.h."""
+    """Load the library (once) and declare every entry point of include/amem.h and include/amem_testing.h."""
     global _lib
     if _lib is not None:
         return _lib
@@ -156,7 +162,7 @@ def load(path=None):
             "%s is missing: build it with `python asystem-amem_amd/build.py` "
             "(there is no Python or CPU fallback for the pause/resume path)" % path)
     lib = C.CDLL(path, mode=C.RTLD_GLOBAL)
-    for name, (res, args) in _SIGNATURES.items():
+    for name, (res, args) in list(_SIGNATURES.items()) + list(_TESTING_SIGNATURES.items()):
         fn = getattr(lib, name)
         fn.restype = res
         fn.argtypes = args
@@ -166,3 +172,7 @@ def load(path=None):
 
 def c_abi_names():
     return sorted(_SIGNATURES)
+
+
+def testing_abi_names():
+    return sorted(_TESTING_SIGNATURES)

@@ -6,10 +6,15 @@
 #include <string.h>
 #include <unistd.h>
 
+#include <algorithm>
+#include <chrono>
+#include <vector>
+
 #include <hip/hip_runtime_api.h>
 
 #include "../../include/amem.h"
 #include "../../include/amem_nccl.h"
+#include "../../include/amem_testing.h"
 #include "ctx.h"
 #include "engine.h"
 #include "ipc.h"
@@ -650,6 +655,7 @@ static OptRef* opt_table(size_t* n) {
       {"pool_limit_bytes", &o.pool_limit_bytes, 0, (int64_t)1 << 46},
       {"scratch_on_host", &o.scratch_on_host, 0, 1},
       {"release_thread", &o.release_thread, 0, 1},
+      {"pause_adaptive", &o.pause_adaptive, 0, 1},
   };
   *n = sizeof(t) / sizeof(t[0]);
   return t;
@@ -791,6 +797,53 @@ int amem_device_mem_info(uint64_t* free_bytes, uint64_t* total_bytes) {
   return e;
 }
 int amem_device_count(void) { return gpu_present() ? g_device_count : 0; }
+int amem_device_pci_bus_id(char* out, int len) {
+  if (int e = need_gpu("amem_device_pci_bus_id")) return e;
+  if (!out || len < 13) return 1;
+  return (int)CHECK_HIP(hipDeviceGetPCIBusId(out, len, current_device()));
+}
+int amem_probe_unmap(int count, uint64_t bytes, double* unmap_us_p50, double* unmap_us_mean, double* map_us_mean) {
+  if (int e = need_gpu("amem_probe_unmap")) return e;
+  if (count < 1 || count > 4096 || bytes == 0) return 1;
+  const int dev = current_device();
+  struct M { uint64_t va, handle; size_t size; };
+  std::vector<M> maps;
+  hipError_t e = hipSuccess;
+  // addresses first, so that the timed triple is what a resume does: create, map, grant access
+  for (int i = 0; i < count && e == hipSuccess; ++i) {
+    void* ptr = nullptr;
+    const size_t size = (bytes + kVmmAlign - 1) / kVmmAlign * kVmmAlign;
+    e = CHECK_HIP(hipMemAddressReserve(&ptr, size, kVmmAlign, nullptr, 0));
+    if (e == hipSuccess) maps.push_back({(uint64_t)(uintptr_t)ptr, 0, size});
+  }
+  double map_us = 0;
+  size_t mapped = 0;
+  for (; mapped < maps.size() && e == hipSuccess; ++mapped) {
+    const auto t0 = std::chrono::steady_clock::now();
+    e = vmm_create_map(maps[mapped].va, dev, maps[mapped].size, &maps[mapped].handle);
+    map_us += std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+    if (e != hipSuccess) break;
+  }
+  (void)CHECK_HIP(hipDeviceSynchronize());
+  std::vector<double> us;
+  for (size_t i = 0; i < mapped; ++i) {
+    const auto t0 = std::chrono::steady_clock::now();
+    hipError_t e2 = vmm_unmap(maps[i].va, maps[i].size);
+    us.push_back(std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count());
+    if (e == hipSuccess) e = e2;
+  }
+  for (size_t i = 0; i < mapped; ++i) (void)vmm_release(maps[i].handle, 0);
+  for (const M& m : maps) (void)hipMemAddressFree((void*)(uintptr_t)m.va, m.size);
+  if (!us.empty()) {
+    double sum = 0;
+    for (double v : us) sum += v;
+    std::sort(us.begin(), us.end());
+    if (unmap_us_p50) *unmap_us_p50 = us[us.size() / 2];
+    if (unmap_us_mean) *unmap_us_mean = sum / us.size();
+    if (map_us_mean) *map_us_mean = map_us / us.size();
+  }
+  return (int)e;
+}
 
 }  // extern "C"
 

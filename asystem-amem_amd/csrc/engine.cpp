@@ -602,6 +602,7 @@ hipError_t Engine::pause_copy_interleaved(Ctx& c, std::vector<Region*>& regs) {
   const bool split = options().release_thread != 0;
   std::vector<std::pair<uint64_t, int>> to_release(split ? n : 0);
   std::atomic<size_t> unmapped{0};
+  std::atomic<size_t> groups_unmapped{0};
   std::atomic<bool> unmapper_done{false};
   auto tc = Clock::now();
   std::thread unmapper([&] {
@@ -619,6 +620,7 @@ hipError_t Engine::pause_copy_interleaved(Ctx& c, std::vector<Region*>& regs) {
         if (e2 != hipSuccess) { failed.store((int)e2); break; }
       }
       if (failed.load()) break;
+      groups_unmapped.store(g + 1, std::memory_order_release);
     }
     unmapper_done.store(true, std::memory_order_release);
   });
@@ -639,12 +641,36 @@ hipError_t Engine::pause_copy_interleaved(Ctx& c, std::vector<Region*>& regs) {
   });
   (void)CHECK_HIP(hipEventRecord(start, kstream_));
   e = hipSuccess;
+  // Adaptive width (option pause_adaptive, on by default). The copy needs less time than the unmaps
+  // (146 ms against 160-175 ms for the 10 GiB training-rank footprint), and an unmap costs less beside a
+  // narrower kernel (measured in one process, cycle by cycle: 295 us beside 8 workgroups, 292 beside 5-7,
+  // 279 beside 4, 235-245 with nothing running; 5 workgroups already saturate the link, 4 copy at 44 GB/s).
+  // So the launcher keeps only a few launches queued, looks at how many finished groups still wait to be
+  // unmapped, and gives up copy rate it does not need: 6 workgroups when the copy is more than 8 groups
+  // ahead, 4 beyond 16, the full width again once the lead is under 4 groups. Where the copy is the
+  // longer of the two (few large regions) the lead never builds up and nothing changes. Measured on two
+  // machines: pause 172.5 -> 164.7 ms and 174.1 -> 165.7 ms; fixed widths of 5, 6, 7 and 12 workgroups
+  // 170-174 ms, a fixed 4 169-172 ms (then the copy is the longer one), and limiting the queue depth
+  // without narrowing changes nothing (173 ms).
+  const bool adaptive = options().pause_adaptive != 0 && shape.xcds == 1 && shape.wgs > 4;
+  constexpr size_t kDepth = 4;
+  uint32_t wgs = shape.wgs;
   for (size_t g = 0; g < groups.size(); ++g) {
     const Group& G = groups[g];
+    if (adaptive && g >= kDepth) {
+      e = CHECK_HIP(hipEventSynchronize(events_[ev0 + g - kDepth]));
+      if (e != hipSuccess) break;
+      const size_t copied = g - kDepth + 1, gone = groups_unmapped.load(std::memory_order_acquire);
+      const size_t lead = copied > gone ? copied - gone : 0;
+      if (lead > 16) wgs = 4;
+      else if (lead > 8) wgs = std::min<uint32_t>(shape.wgs, 6);
+      else if (lead < 4) wgs = shape.wgs;
+      if (wgs != shape.wgs) stats_.pause_narrow_launches++;
+    }
     if (G.d1 > G.d0 && tp[G.d1] > tp[G.d0]) {
       e = CHECK_HIP(launch_move(false, (const CopyDesc*)d_descs_.p + G.d0, (const uint64_t*)d_tiles_.p + G.d0,
                                 G.d1 - G.d0, tp[G.d0], tp[G.d1] - tp[G.d0], pool_tab, 0,
-                                shape.wgs, shape.xcds, kstream_));
+                                wgs, shape.xcds, kstream_));
       if (e != hipSuccess) break;
       stats_.k2_launches++;
       stats_.kernel_bytes += G.bytes;

@@ -35,6 +35,7 @@ struct Options {
   int64_t resume_dma_min_bytes = 0;       // resume: runs this long come back by hipMemcpyAsync on the second stream (0 = none)
   int64_t peer_timeout_ms = 60000;
   int64_t release_thread = 1;             // interleaved path: handles are released on a third thread
+  int64_t pause_adaptive = 1;             // interleaved path: narrow the gather kernel while the copy runs ahead of the unmaps
   int64_t scratch_on_host = 0;            // 1: engine tables live in pinned host memory even if the device has room
   int64_t pool_limit_bytes = 0;           // cap on pinned host memory a pause may need, 0 = none
   int64_t offload_free_tag = -1;          // caller tag whose regions are released without being copied

@@ -17,7 +17,11 @@ Prints one JSON line:
   link_kernels  the two kernels that take nearly all GPU time, gather-pack and scatter-unpack against pinned
              host memory: bytes per leg, device time, GB/s, fraction of the measured link rate
   first_cycle  times and phases of the very first cycle (pinned pool and engine tables are created in it)
-  unmap      what the unmapping thread spends per region (the sum bounds the pause)
+  unmap      what the unmapping thread spends per region (the sum bounds the pause), what one hipMemUnmap costs
+             on this machine with nothing else running (idle_us, probed before the timed cycles), the floor
+             regions x idle_us + scan + plan that no pause of this footprint can beat, and pause_over_floor
+  other_configs  configurations 1, 2 and 4 timed the same way for a few cycles each after the headline
+  host       where the pinned slabs sit (NUMA node) beside the GPU's own node
   pack_unpack_in_hbm  the pack and unpack kernels with both sides in HBM, against HBM peak
   reference_structure_on_gpu  the reference's loop structure in HIP calls on the same footprint
   cpu_baseline  the reference's serial per-region memcpy path (oracle/) on this box's host cores,
@@ -84,6 +88,75 @@ def cpu_baseline(threads_all, gib):
             "all_cores": {"value": round(out[threads_all], 3), "cores": threads_all}}
 
 
+def numa_placement(lib, slab_addr):
+    """NUMA node of one pinned slab page beside the GPU's node (sysfs). The reference places its host buffers
+    on the GPU's node by hand with an explicit fallback (amem_nccl.h:251-267); here the runtime places them."""
+    out = {"nodes_online": None, "gpu_numa_node": None, "slab_numa_node": None}
+    try:
+        out["nodes_online"] = open("/sys/devices/system/node/online").read().strip()
+    except OSError:
+        pass
+    bdf = C.create_string_buffer(32)
+    if lib.amem_device_pci_bus_id(bdf, 32) == 0:
+        try:
+            out["gpu_pci"] = bdf.value.decode().lower()
+            out["gpu_numa_node"] = int(open("/sys/bus/pci/devices/%s/numa_node" % out["gpu_pci"]).read())
+        except (OSError, ValueError):
+            pass
+    if slab_addr:
+        try:
+            libc = C.CDLL(None, use_errno=True)
+            page = C.c_void_p(slab_addr & ~4095)
+            status = C.c_int(-999)
+            # move_pages(pid 0, one page, no target nodes) only reports where the page is (syscall 279 on x86-64)
+            rc = libc.syscall(279, 0, C.c_ulong(1), C.byref(page), None, C.byref(status), 0)
+            if rc == 0 and status.value >= 0:
+                out["slab_numa_node"] = status.value
+            else:
+                out["slab_numa_node_unknown"] = ("move_pages rc %d status %d errno %d: the kernel does not report a node for "
+                                                 "this kind of mapping" % (rc, status.value, C.get_errno()))
+        except Exception as e:  # noqa: BLE001 - a diagnostic must not break the benchmark
+            out["slab_numa_node_unknown"] = repr(e)
+    if out["nodes_online"] is not None and "-" not in out["nodes_online"] and "," not in out["nodes_online"]:
+        out["note"] = "this machine has a single NUMA node: placement cannot be wrong"
+    return out
+
+
+def time_config(lib, B, H, fp, warmup, steps, d2h, h2d):
+    """One footprint through `warmup` untimed and `steps` timed pause/resume cycles, with the correctness gate."""
+    regs = H.Regions(lib, fp)
+    F = int(regs.alloc.sum())
+    va_before, table_before = regs.va.copy(), regs.table()
+    pause_s, resume_s, stats = [], [], []
+    for step in range(warmup + steps):
+        if hasattr(fp, "mutate"):
+            regs.write_chunks(fp.mutate(1000 + step))
+        t0 = time.perf_counter()
+        rc1 = lib.amem_mem_pause(0, 0)
+        t1 = time.perf_counter()
+        rc2 = lib.amem_mem_resume(0, 0)
+        t2 = time.perf_counter()
+        assert rc1 == 0 and rc2 == 0, (rc1, rc2)
+        if step >= warmup:
+            pause_s.append(t1 - t0); resume_s.append(t2 - t1); stats.append(H.cycle_stats(lib))
+    bad = regs.mismatched_bytes()
+    tdiff = [d for d in H.compare_tables(table_before, regs.table()) if d[1] != "handle_gen"]
+    ok = bad == 0 and bool((regs.va == va_before).all()) and not tdiff
+    n = len(fp.sizes)
+    regs.free()
+    lib.amem_pool_trim()
+    pp, pr = statistics.median(pause_s), statistics.median(resume_s)
+    parked = statistics.mean(s["parked_bytes"] for s in stats)
+    return {"regions": n, "footprint_bytes": F, "parked_bytes_per_leg": int(parked), "cycles_timed": steps,
+            "p50_pause_s": round(pp, 5), "p50_resume_s": round(pr, 5),
+            "effective_GBps": round(2 * F / (pp + pr) / 1e9, 2),
+            "pause_leg_frac_of_link": round(parked / pp / 1e9 / d2h, 4),
+            "resume_leg_frac_of_link": round(parked / pr / 1e9 / h2d, 4),
+            "pause_us_per_region": round(pp * 1e6 / n, 1), "resume_us_per_region": round(pr * 1e6 / n, 1),
+            "unmap_us_each_p50": round(statistics.median(s["pause_unmap_ms"] for s in stats) * 1e3 / n, 1),
+            "bit_exact": ok}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -96,6 +169,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-reference-structure", action="store_true")
     ap.add_argument("--no-hbm-kernels", action="store_true", help="skip the pack/unpack-in-HBM measurement")
+    ap.add_argument("--no-other-configs", action="store_true", help="skip the short runs of configurations 1, 2 and 4")
     ap.add_argument("--pause-path", type=int, default=None)
     ap.add_argument("--opt", action="append", default=[], help="engine tunable, name=value (see amem_set_option)")
     ap.add_argument("--calib", action="store_true",
@@ -130,6 +204,11 @@ def main():
     if args.calib:
         ms = C.c_float()
         assert lib.amem_calib_copy(1 << 30, 3, C.byref(ms)) == 0
+
+    # What one hipMemUnmap costs here with nothing running: 64 mappings of 2 MiB, accessible, device idle.
+    idle_p50, idle_mean, map_mean = C.c_double(), C.c_double(), C.c_double()
+    assert lib.amem_probe_unmap(64, 2 << 20, C.byref(idle_p50), C.byref(idle_mean), C.byref(map_mean)) == 0
+    assert lib.amem_probe_unmap(64, 2 << 20, C.byref(idle_p50), C.byref(idle_mean), C.byref(map_mean)) == 0  # (second pass: warm)
 
     if args.config == 3:
         fp = Footprint(3, 2, byte_budget=int(args.gib * (1 << 30)), threads=host_threads)
@@ -214,6 +293,9 @@ def main():
                                "workgroup) with a device-side buffer: 2*S bytes (S read + S written) per launch, "
                                "p50 of 3 launches after a warm one; the bytes are checked afterwards with the rest"}
 
+    slab_addr = next((t["cpu_addr"] for t in regs.table().values() if t["cpu_addr"]), 0)
+    numa = numa_placement(lib, slab_addr)
+
     # correctness gate, outside the clock: bytes, addresses, table
     bad = regs.mismatched_bytes()
     same_va = bool((regs.va == va_before).all())
@@ -243,6 +325,8 @@ def main():
     k3_ms = statistics.median(s["k3_ms"] for s in stats)
     kbytes = statistics.mean(s["kernel_bytes"] for s in stats)
     PCIE_GEN5_X16 = 63.0
+    pause_floor = (len(fp.sizes) * idle_p50.value * 1e-6 +
+                   statistics.median(s["pause_scan_ms"] + s["pause_plan_ms"] + s["pause_sync_ms"] for s in stats) * 1e-3)
     pause_frac = parked / p50_pause / 1e9 / d2h.value
     resume_frac = parked / p50_resume / 1e9 / h2d.value
     out = {
@@ -308,10 +392,17 @@ def main():
                     "these two kernels are over 99 % of the GPU time of a cycle, the scan kernel of `roofline` under 1 %"},
         "unmap": {"regions": len(fp.sizes), "us_each_p50": round(statistics.median(s["pause_unmap_ms"] for s in stats)
                                                                    * 1e3 / max(len(fp.sizes), 1), 1),
-                  "what": "time the unmapping thread spends per region (hipMemUnmap beside the gather kernel); "
-                          "the sum bounds the pause"},
+                  "idle_us": round(idle_p50.value, 1), "idle_us_mean": round(idle_mean.value, 1),
+                  "create_map_access_us": round(map_mean.value, 1),
+                  "pause_floor_s": round(pause_floor, 4), "pause_over_floor": round(p50_pause / pause_floor, 3),
+                  "what": "us_each_p50: time the unmapping thread spends per region (hipMemUnmap beside the gather kernel); "
+                          "the sum bounds the pause. idle_us: one hipMemUnmap of an accessible 2 MiB mapping with nothing else "
+                          "running, p50 of 64, probed before the timed cycles. pause_floor_s = regions x idle_us + scan + "
+                          "plan + sync: every mapping has to be unmapped inside the pause and the runtime serialises the calls. "
+                          "pause_over_floor = p50_pause_s / pause_floor_s"},
         "phases_ms_p50": {k: round(statistics.median(s[k] for s in stats), 3) for k in PHASES},
-        "host": {"cpus_reported": host_cpus, "threads_used": host_threads},
+        "host": dict({"cpus_reported": host_cpus, "threads_used": host_threads},
+                     **{k: v for k, v in numa.items()}),
     }
     if hbm_kernels:
         out["pack_unpack_in_hbm"] = hbm_kernels
@@ -319,6 +410,23 @@ def main():
         out["reference_structure_on_gpu"] = ref_struct
         out["speedup_vs_reference_structure"] = round(out["value"] / ref_struct["value"], 3)
     regs.free()
+    lib.amem_pool_trim()
+    if not args.no_other_configs and args.config == 3:
+        from asystem_amem_amd.footprint import PackedGranules
+        others = {}
+        for name, make in (("config_1", lambda: Footprint(1, 0, threads=host_threads)),
+                           ("config_2", lambda: Footprint(2, 1, threads=host_threads)),
+                           ("config_4", lambda: PackedGranules(3, 100000, threads=host_threads))):
+            others[name] = time_config(lib, B, H, make(), 1, 5, d2h.value, h2d.value)
+            ok = ok and others[name]["bit_exact"]
+        others["what"] = ("the other single-process configurations of the benchmark, 5 timed cycles each after a warm one, "
+                          "1 % of chunks rewritten between cycles where the footprint has a generator for it: config 1 = 64 "
+                          "regions of 2 MiB x U{1..16}, no zero chunks, seed 0; config 2 = inference rank, 128x4 + 96x2 + 32x16 "
+                          "MiB, 50 % zero chunks, seed 1; config 4 = 100,000 sub-allocations of 4-64 KiB packed into 2 MiB "
+                          "granules, every granule one region, seed 3. Pause time follows the number of regions (one "
+                          "hipMemUnmap each), not the bytes")
+        out["other_configs"] = others
+        out["bit_exact"] = ok
     if not args.no_cpu_baseline and args.config == 3:
         out["cpu_baseline"] = cpu_baseline(host_threads, args.gib)
         out["cpu_baseline"]["host_cpus_reported"] = host_cpus

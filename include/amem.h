@@ -260,6 +260,7 @@ typedef struct amem_cycle_stats {
   double pause_sync_ms;     /* of pause_ms: the device synchronisation and memory queries before the scan */
   double resume_scratch_ms; /* of resume_ms: allocating or growing the engine's own tables and events */
   uint64_t resume_dma_bytes; /* of parked_bytes, how much the resume brought back by hipMemcpyAsync */
+  uint64_t pause_narrow_launches; /* of k2_launches, how many "pause_adaptive" issued with fewer workgroups */
 } amem_cycle_stats;
 void amem_get_cycle_stats(amem_cycle_stats* out);
 
@@ -311,6 +312,10 @@ int amem_set_enabled(int on);
  *                     option's initial value when the library is loaded (a WARN line says so)
  *   "release_thread"  0/1 (default 1): the default pause path releases handles on a thread of their own
  *                     instead of on the one that unmaps
+ *   "pause_adaptive"  0/1 (default 1): the default pause path keeps only a few launches queued and issues
+ *                     them with 6 or 4 workgroups instead of "pause_wgs" while finished groups pile up
+ *                     in front of the unmapping thread: an unmap costs less beside a narrower kernel, and
+ *                     the copy has time to spare when there are many regions. 0 = every launch "pause_wgs" wide
  *   "scratch_on_host" 0/1: keep the engine's own tables in pinned host memory. That is where they go
  *                     anyway when the device has no room for them at pause time; 1 forces it
  *   "pool_limit_bytes" most pinned host memory one pause may need (0 = no limit). A pause that
@@ -383,14 +388,17 @@ uint64_t amem_chunk_count(const amem_extent* extents, uint64_t n);
 int amem_zero_scan(const amem_extent* extents, uint64_t n, uint8_t* flags,
                    amem_chunk_sum* sums, float* kernel_ms);
 
-/* amem_zero_scan for callers that cannot allocate device memory (code under HIP graph capture,
- * tight serving loops, harnesses that forbid it). No counterpart in the reference. Same arguments
- * and bit-identical results; the tables the scan kernel needs beyond its inputs and outputs
- * (segment table, chunk prefix, flags and checksums before they reach the host) live in one fixed
- * device array of about 4.4 MiB that every GPU the library runs on holds until the process ends,
- * and the host side of every transfer is pinned memory made when the device's engine is set up
- * (by the first tracked allocation, or by the first call of any entry point of this section on
- * that device). After that set-up a call allocates and frees nothing, on the device or the host.
+/* amem_zero_scan for callers that cannot allocate device memory (tight serving loops, harnesses
+ * that forbid hipMalloc). No counterpart in the reference. Same arguments and bit-identical
+ * results; the tables the scan kernel needs beyond its inputs and outputs (segment table, chunk
+ * prefix, flags and checksums before they reach the host) live in one fixed device array of about
+ * 4.4 MiB that every GPU the library runs on holds until the process ends, and the host side of
+ * every transfer is pinned memory made when the device's engine is set up (by the first tracked
+ * allocation, or by the first call of any entry point of this section on that device: make one
+ * warm-up call first). After that set-up a call allocates and frees nothing, on the device or the
+ * host. It is serialised with every other engine call on the engine's lock, enqueues its copies and
+ * its kernel on the engine's own stream and synchronises that stream before it returns: call it
+ * outside any stream capture.
  * Limits: at most AMEM_NOALLOC_MAX_EXTENTS extents and AMEM_NOALLOC_MAX_CHUNKS chunks (16 GiB)
  * per call; beyond them the call logs the limit and returns hipErrorInvalidValue (1) without
  * touching the GPU. All calls on one GPU share the fixed array, which keeps the last call's
@@ -418,20 +426,6 @@ int amem_gather_pack(const amem_copy_desc* descs, uint64_t n, void* staging,
                      uint64_t staging_bytes, int host_side, float* kernel_ms);
 int amem_scatter_unpack(const amem_copy_desc* descs, uint64_t n, const void* staging,
                         uint64_t staging_bytes, int host_side, float* kernel_ms);
-
-/* Measured host-link roofline: best-of-`reps` hipMemcpy of `bytes` between device memory
- * and a pinned host buffer, each direction, in GB/s (1e9 bytes per second). */
-int amem_probe_link(uint64_t bytes, int reps, double* d2h_gbps, double* h2d_gbps);
-
-/* Plain device-to-device copy kernel of `bytes` (multiple of 16), used to calibrate the
- * FETCH_SIZE / WRITE_SIZE hardware counters against a known traffic. */
-int amem_calib_copy(uint64_t bytes, int reps, float* kernel_ms);
-
-/* Raw byte access for tests and benchmarks (hipMemcpy wrappers, synchronous). */
-int amem_copy_to_device(uint64_t va, const void* host, uint64_t bytes);
-int amem_copy_from_device(void* host, uint64_t va, uint64_t bytes);
-int amem_device_mem_info(uint64_t* free_bytes, uint64_t* total_bytes);
-int amem_device_count(void);
 
 #pragma GCC visibility pop
 #ifdef __cplusplus

@@ -17,6 +17,7 @@
 #include <vector>
 
 #include "../../include/amem.h"
+#include "../../include/amem_testing.h"
 
 static std::atomic<long> g_errors{0};
 #define EXPECT(x) do { if (!(x)) { g_errors++; fprintf(stderr, "EXPECT failed line %d: %s\n", __LINE__, #x); } } while (0)

@@ -1,8 +1,10 @@
-/* A plain C99 caller of the C ABI: proves that include/amem.h is valid C and that the symbols link. */
+/* A plain C99 caller of the C ABI: proves that include/amem.h and include/amem_testing.h are valid C
+ * and that the symbols link. */
 #include <stdio.h>
 #include <stdlib.h>
 
 #include "amem.h"
+#include "amem_testing.h"
 
 int main(void) {
   amem_counters c;
@@ -21,6 +23,7 @@ int main(void) {
   if (ncclMemStats() != 0 || ncclGetGroupID(&gid) != 0) return 9;
   if (amem_del_alloc_info(0x7f0000000000ull, 0xabcull, 0) != 0 || amem_region_count(0) != 0) return 10;
   if (amem_shutdown() != 0) return 11;
+  if (amem_device_count() < 0) return 12; /* a helper of amem_testing.h: 0 without a GPU */
   printf("c caller ok\n");
   return 0;
 }

@@ -36,6 +36,10 @@ def test_library_exports_every_declared_symbol(lib):
     missing = sorted(d for d in declared if d not in syms)
     assert not missing, missing
     assert set(B.c_abi_names()) == declared, set(B.c_abi_names()) ^ declared
+    # the measurement and test helpers have a header of their own and are not part of the product surface
+    helpers = declared_c_functions("amem_testing.h")
+    assert helpers and not (helpers & declared) and all(h in syms for h in helpers)
+    assert set(B.testing_abi_names()) == helpers, set(B.testing_abi_names()) ^ helpers
     # the reference's C++-linkage names, exactly as its library exports them
     for m in B.MANGLED_REFERENCE_SYMBOLS:
         assert m in syms, m
@@ -236,8 +240,8 @@ def test_memstats_output_matches_readme_sample():
 
 
 def test_headers_compile_and_link_from_c_and_cxx(tmp_path):
-    """include/amem.h is valid C99 for a C compiler, include/amem_nccl.h gives C++ callers the
-    reference's API; both link against the built library and run (registry calls only)."""
+    """include/amem.h and include/amem_testing.h are valid C99 for a C compiler, include/amem_nccl.h gives
+    C++ callers the reference's API; all link against the built library and run (registry calls only)."""
     inc, libdir = os.path.join(ROOT, "include"), os.path.dirname(B.LIB_PATH)
     env = dict(os.environ, AMEM_ENABLE="1", GMM_LOG="1", AMEM_IPC="0", LD_LIBRARY_PATH=libdir + ":" + os.environ.get("LD_LIBRARY_PATH", ""))
     for compiler, std, src, exe in (("gcc", "-std=c99", "c_caller.c", "c_caller"),
@@ -260,7 +264,8 @@ def test_rccl_hook_library_exports_the_interposed_calls():
     names = {l.split()[-1] for l in out.splitlines() if " T " in l}
     assert names == {"hipMemMap", "hipMemSetAccess", "hipMemUnmap", "hipMemImportFromShareableHandle",
                      "hipMemExportToShareableHandle", "hipMemRelease", "hipMalloc", "hipFree", "hipExtMallocWithFlags",
-                     "amem_rccl_hook_registered", "amem_rccl_hook_served_bytes"}
+                     "hipIpcGetMemHandle", "amem_rccl_hook_registered", "amem_rccl_hook_served_bytes",
+                     "amem_rccl_hook_unserved_bytes", "amem_rccl_hook_exclude"}
     # unversioned definitions: they satisfy librccl's versioned references (hipMemMap@hip_5.1 ...)
     assert "@" not in "".join(names)
 

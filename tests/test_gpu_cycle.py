@@ -21,7 +21,8 @@ GiB = 1 << 30
 def eng(gpu, fresh):
     defaults = {k: fresh.amem_get_option(k) for k in (b"zero_elide", b"verify", b"pause_path", b"dma_min_bytes",
                                                        b"staging_bytes", b"resume_batch_bytes", b"scratch_on_host", b"release_thread",
-                                                       b"pause_wgs", b"pause_xcds", b"interleave_bytes", b"resume_dma_min_bytes")}
+                                                       b"pause_wgs", b"pause_xcds", b"interleave_bytes", b"resume_dma_min_bytes",
+                                                       b"pause_adaptive")}
     yield fresh
     fresh.amem_mem_resume(0, 0)        # a test that failed mid-cycle must not leave the engine paused
     for k, v in defaults.items():
@@ -128,6 +129,7 @@ def test_repeated_cycles_with_writes_between(eng):
                                   {"staging_bytes": 1 << 20, "resume_batch_bytes": 1 << 40},
                                   {"pause_path": 3, "interleave_bytes": 1 << 16}, {"pause_path": 4},
                                   {"release_thread": 0}, {"release_thread": 0, "pause_wgs": 96, "pause_xcds": 8},
+                                  {"pause_adaptive": 0}, {"pause_adaptive": 1, "interleave_bytes": 1 << 16},
                                   {"resume_dma_min_bytes": 128 << 10}, {"resume_dma_min_bytes": 1 << 16, "pause_path": 0, "dma_min_bytes": 128 << 10},
                                   {"resume_dma_min_bytes": 1 << 16, "zero_elide": 0}])
 def test_option_paths_are_all_bit_exact(eng, opts):
