@@ -15,10 +15,11 @@ Prints one JSON line:
   roofline   the on-device scan kernel (zero flags + checksums) against HBM peak
   link       each leg against the measured hipMemcpy rate of the host link
   link_kernels  the two kernels that take nearly all GPU time, gather-pack and scatter-unpack against pinned
-             host memory: bytes per leg, device time, GB/s, fraction of the measured link rate
+             host memory: bytes per leg, device time, GB/s, fraction of the measured link rate (the gather
+             kernel is narrowed on purpose while the copy runs ahead of the unmaps: launches_narrowed)
   first_cycle  times and phases of the very first cycle (pinned pool and engine tables are created in it)
   unmap      what the unmapping thread spends per region (the sum bounds the pause), what one hipMemUnmap costs
-             on this machine with nothing else running (idle_us, probed before the timed cycles), the floor
+             on this machine with nothing else running (idle_us, probed before and after the timed cycles), the floor
              regions x idle_us + scan + plan that no pause of this footprint can beat, and pause_over_floor
   other_configs  configurations 1, 2 and 4 timed the same way for a few cycles each after the headline
   host       where the pinned slabs sit (NUMA node) beside the GPU's own node
@@ -293,6 +294,9 @@ def main():
                                "workgroup) with a device-side buffer: 2*S bytes (S read + S written) per launch, "
                                "p50 of 3 launches after a warm one; the bytes are checked afterwards with the rest"}
 
+    # the same probe again after the timed cycles: the cost of the call drifts on these machines
+    idle_after = C.c_double()
+    assert lib.amem_probe_unmap(64, 2 << 20, C.byref(idle_after), None, None) == 0
     slab_addr = next((t["cpu_addr"] for t in regs.table().values() if t["cpu_addr"]), 0)
     numa = numa_placement(lib, slab_addr)
 
@@ -325,7 +329,8 @@ def main():
     k3_ms = statistics.median(s["k3_ms"] for s in stats)
     kbytes = statistics.mean(s["kernel_bytes"] for s in stats)
     PCIE_GEN5_X16 = 63.0
-    pause_floor = (len(fp.sizes) * idle_p50.value * 1e-6 +
+    idle_us = min(idle_p50.value, idle_after.value)
+    pause_floor = (len(fp.sizes) * idle_us * 1e-6 +
                    statistics.median(s["pause_scan_ms"] + s["pause_plan_ms"] + s["pause_sync_ms"] for s in stats) * 1e-3)
     pause_frac = parked / p50_pause / 1e9 / d2h.value
     resume_frac = parked / p50_resume / 1e9 / h2d.value
@@ -378,8 +383,9 @@ def main():
                  "resume_copy_phase_frac": round(parked / (statistics.median(s["resume_copy_ms"] for s in stats) * 1e-3)
                                                  / 1e9 / h2d.value, 4)},
         "link_kernels": {
-            "move_tiles<0> (gather-pack into pinned host memory, 8 workgroups on one XCD, unmaps running beside it)": {
+            "move_tiles<0> (gather-pack into pinned host memory, 4 to 8 workgroups on one XCD, unmaps running beside it)": {
                 "bound": "host link D2H", "bytes_per_pause": int(kbytes), "launches_per_pause": int(statistics.median(s["k2_launches"] for s in stats)),
+                "launches_narrowed": int(statistics.median(s["pause_narrow_launches"] for s in stats)),
                 "device_ms_per_pause": round(k2_ms, 3), "GBps": round(kbytes / k2_ms / 1e6, 2) if k2_ms else None,
                 "frac_of_measured_d2h": round(kbytes / k2_ms / 1e6 / d2h.value, 4) if k2_ms else None,
                 "frac_of_pcie_gen5_x16": round(kbytes / k2_ms / 1e6 / PCIE_GEN5_X16, 4) if k2_ms else None},
@@ -392,12 +398,12 @@ def main():
                     "these two kernels are over 99 % of the GPU time of a cycle, the scan kernel of `roofline` under 1 %"},
         "unmap": {"regions": len(fp.sizes), "us_each_p50": round(statistics.median(s["pause_unmap_ms"] for s in stats)
                                                                    * 1e3 / max(len(fp.sizes), 1), 1),
-                  "idle_us": round(idle_p50.value, 1), "idle_us_mean": round(idle_mean.value, 1),
+                  "idle_us": round(idle_us, 1), "idle_us_before": round(idle_p50.value, 1), "idle_us_after": round(idle_after.value, 1),
                   "create_map_access_us": round(map_mean.value, 1),
                   "pause_floor_s": round(pause_floor, 4), "pause_over_floor": round(p50_pause / pause_floor, 3),
                   "what": "us_each_p50: time the unmapping thread spends per region (hipMemUnmap beside the gather kernel); "
                           "the sum bounds the pause. idle_us: one hipMemUnmap of an accessible 2 MiB mapping with nothing else "
-                          "running, p50 of 64, probed before the timed cycles. pause_floor_s = regions x idle_us + scan + "
+                          "running, p50 of 64, probed before and after the timed cycles (the lower of the two). pause_floor_s = regions x idle_us + scan + "
                           "plan + sync: every mapping has to be unmapped inside the pause and the runtime serialises the calls. "
                           "pause_over_floor = p50_pause_s / pause_floor_s"},
         "phases_ms_p50": {k: round(statistics.median(s[k] for s in stats), 3) for k in PHASES},
