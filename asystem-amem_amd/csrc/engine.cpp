@@ -1280,9 +1280,18 @@ int Engine::resume(Ctx& c, bool* incomplete) {
     e = vmm_export_fd(x.handle, &fd);
     note(e);
     if (e != hipSuccess) continue;
+    // every importer of the region is told at once (the reference tells them one after the other,
+    // amem_nccl.cpp:636-645): they import and map side by side
+    int slots[AMEM_MAX_DEVS], rets[AMEM_MAX_DEVS], nslots = 0;
+    uint64_t vas[AMEM_MAX_DEVS];
     for (int s = 0; s < AMEM_MAX_DEVS; ++s) {
       if (peers[s] == 0) continue;
-      int ret = peer_update(s, peers[s], fd);
+      slots[nslots] = s;
+      vas[nslots++] = peers[s];
+    }
+    peer_update_many(slots, vas, nslots, fd, rets);
+    for (int k = 0; k < nslots; ++k) {
+      const int s = slots[k], ret = rets[k];
       if (ret != 0 && !peer_alive(s)) {
         // The importer's process is gone and its mapping with it: nothing to update, now or later.
         LOGGER(WARN, "groupID:%d pid:%d localDptr:%llx the importer in slot %d is gone, forgetting its mapping %llx",
@@ -1290,7 +1299,7 @@ int Engine::resume(Ctx& c, bool* incomplete) {
         std::lock_guard<std::mutex> lk(c.fields);
         x.r->peers[s] = 0;
         x.r->hasPeer = false;
-        for (int k = 0; k < AMEM_MAX_DEVS; ++k) x.r->hasPeer |= x.r->peers[k] != 0;
+        for (int j = 0; j < AMEM_MAX_DEVS; ++j) x.r->hasPeer |= x.r->peers[j] != 0;
         c.releaseLocalCnt--;
       } else if (ret != 0) {
         LOGGER(ERROR, "groupID:%d pid:%d localDptr:%llx newHandle:%llx fd:%d notify peer %d to remap dptr:%llx ret:%d",

@@ -449,6 +449,58 @@ int peer_register(uint64_t src_handle, uint64_t my_va, int owner_slot) {
   return ret;
 }
 
+// One descriptor to several importers at once: every request goes out before the first answer is
+// waited for, so the importers (one service thread each, usually one process each) import and map side
+// by side instead of one after the other. Slots are taken in ascending order, each connection stays
+// locked from its request to its answer.
+void peer_update_many(const int* slots, const uint64_t* peer_vas, int n, int fd, int* rets) {
+  int socks[AMEM_MAX_DEVS];
+  bool locked[AMEM_MAX_DEVS];
+  bool mine[AMEM_MAX_DEVS];
+  if (n > AMEM_MAX_DEVS) n = AMEM_MAX_DEVS;
+  // (asked before any connection is locked: own_slot takes the lock that ipc_stop holds while it
+  // takes the connections' locks)
+  for (int i = 0; i < n; ++i) mine[i] = own_slot(slots[i]);
+  for (int i = 0; i < n; ++i) {
+    socks[i] = -1;
+    locked[i] = false;
+    rets[i] = 1;
+    const int slot = slots[i];
+    if (slot < 0 || slot >= AMEM_MAX_DEVS || (i > 0 && slot <= slots[i - 1])) continue;
+    if (mine[i] && !options().peer_loopback) { rets[i] = 0; continue; }
+    if (g_svc.slot < 0) continue;
+    g_ipc.conn_mtx[slot].lock();
+    locked[i] = true;
+    const int s = connect_if_not(slot);
+    if (s < 0) continue;
+    WireReq req = {kMagic, OP_UPDATE_PEER_INFO, g_svc.slot, (int32_t)getpid(), 0, peer_vas[i]};
+    if (send_msg(s, &req, sizeof(req), fd) == (ssize_t)sizeof(req)) {
+      socks[i] = s;
+    } else {
+      close(s);
+      g_ipc.conn[slot] = -1;
+    }
+  }
+  for (int i = 0; i < n; ++i) {
+    if (!locked[i]) continue;
+    const int slot = slots[i];
+    if (socks[i] >= 0) {
+      int32_t ret = 1;
+      if (recv_msg(socks[i], &ret, sizeof(ret), nullptr) == (ssize_t)sizeof(ret)) {
+        rets[i] = ret;
+      } else {
+        // peer gone, or no answer within the timeout: the next request reconnects
+        close(socks[i]);
+        g_ipc.conn[slot] = -1;
+      }
+    }
+    g_ipc.conn_mtx[slot].unlock();
+    if (rets[i] != 0)
+      LOGGER(WARN, "groupID:%d pid:%d peer_dev:%d peer_dptr:%llx newFD:%d send|recv error", amem_groupID_value(),
+             getpid(), slot, (unsigned long long)peer_vas[i], fd);
+  }
+}
+
 int peer_update(int importer_slot, uint64_t peer_va, int fd) {
   if (own_slot(importer_slot) && !options().peer_loopback) return 0;
   if (g_svc.slot < 0) return 1;

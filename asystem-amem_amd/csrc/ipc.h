@@ -41,6 +41,10 @@ int peer_register(uint64_t src_handle, uint64_t my_va, int owner_slot);
 // this process, gmm_client_impl.cpp:512-514).
 int peer_update(int importer_slot, uint64_t peer_va, int fd);
 
+// The same to `n` importers at once (slots strictly ascending): all requests are sent before the first
+// answer is read. rets[i] as peer_update's return for slots[i].
+void peer_update_many(const int* slots, const uint64_t* peer_vas, int n, int fd, int* rets);
+
 // Handler of a peer's request to drop the mapping at `va` (gmm_worker_impl.cpp:392-397).
 int amem_release_peer_mapping(uint64_t va);
 

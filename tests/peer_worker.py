@@ -88,6 +88,7 @@ def _worker(rank, world, ipc_dir, gid, conns, ctrl, lib_path=None, NREG=NREG):
         fds0 = _nfds()
         free0 = H.mem_free(lib)
         ctrl.send(("checked", rank, free0)); assert ctrl.recv() == "go"
+        timings = []
         for cycle in range(2):
             assert lib.amem_mem_pause(0, 0) == 0
             c = H.counters(lib)
@@ -102,6 +103,8 @@ def _worker(rank, world, ipc_dir, gid, conns, ctrl, lib_path=None, NREG=NREG):
             if cycle == 1 and rank == 0:
                 time.sleep(0.3)                        # importers must wait for a late owner, not fail
             assert lib.amem_mem_resume(0, 0) == 0
+            st = H.cycle_stats(lib)
+            timings.append((st["pause_ms"], st["resume_ms"], st["resume_peer_ms"]))
             c = H.counters(lib)
             assert (c["offload_cnt"], c["release_local_cnt"], c["release_shadow_cnt"], c["paused"]) == (0, 0, 0, 0)
             ctrl.send(("resumed", rank)); assert ctrl.recv() == "go"
@@ -127,7 +130,7 @@ def _worker(rank, world, ipc_dir, gid, conns, ctrl, lib_path=None, NREG=NREG):
             lib.amem_vmm_free(va, size, 0)
         regs.free()
         lib.amem_shutdown()
-        ctrl.send(("exit", rank))
+        ctrl.send(("exit", rank, timings))
     except BaseException as e:  # report instead of hanging the barrier
         import traceback
         ctrl.send(("error", rank, traceback.format_exc()))
@@ -162,12 +165,16 @@ def run_world(world, lib_path=None, gid_base=0x6000, nreg=NREG, phase_timeout=12
                     assert msg[0] == phase, msg
                 for r in range(world):
                     ctrls[r][0].send("go")
+            timings = []
             for r in range(world):
                 assert ctrls[r][0].poll(60)
-                assert ctrls[r][0].recv()[0] == "exit"
+                msg = ctrls[r][0].recv()
+                assert msg[0] == "exit"
+                timings.append(msg[2])
             for p in procs:
                 p.join(60)
                 assert p.exitcode == 0
+            return timings          # per rank: (pause ms, resume ms, of which export + notify + wait) of each cycle
         finally:
             for p in procs:
                 if p.is_alive():

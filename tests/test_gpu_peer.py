@@ -438,3 +438,81 @@ def test_config5_every_rank_owns_and_imports_in_one_process(gpu, fresh, measured
         lib.amem_mem_resume(0, 0)
         lib.amem_ipc_act_as(-1)
         assert lib.amem_set_option(b"peer_loopback", 0) == 0
+
+
+def test_more_shared_regions_than_descriptors_may_be_open(gpu, fresh, measured):
+    """This runtime lets a process keep 1,024 exported descriptors open and no more (the 1,025th export
+    fails, and beside 1,024 open ones no imported mapping can be given access; probed with plain HIP calls
+    through amem_vmm_export / amem_vmm_import below). A resume therefore exports each region only when it
+    tells that region's importers and closes the descriptor before the next (as the reference's loop does,
+    amem_nccl.cpp:613, :646): 1,100 owned regions of 2 MiB, each imported once by a second rank of the
+    process, go through two cycles with every byte checked at both addresses."""
+    from asystem_amem_amd import binding as B, harness as H
+    lib = fresh
+    assert lib.amem_set_option(b"peer_loopback", 1) == 0
+    N = 1100
+    try:
+        owner = lib.amem_ipc_start()
+        rank = lib.amem_ipc_claim_slot()
+        assert owner >= 0 and rank >= 0 and rank != owner
+        rng = np.random.default_rng(77)
+        owned, imports, data = [], [], []
+        for i in range(N):
+            va, h, asz = C.c_uint64(), C.c_uint64(), C.c_uint64()
+            assert lib.amem_vmm_alloc(2 * MiB, 0, C.byref(va), C.byref(h), C.byref(asz)) == 0
+            d = rng.integers(0, 256, 4096, dtype=np.uint8)     # one page of its own per region, the rest stays zero
+            assert lib.amem_copy_to_device(va.value + (i % 32) * 65536, d.ctypes.data, 4096) == 0
+            assert lib.amem_add_alloc_info(va.value, asz.value, B.TYPE_LOCAL, 0, h.value, -1, 0, None, B.CALLER_P2P) == 0
+            owned.append((va.value, h.value, asz.value)); data.append(d)
+        # the limit itself, with nothing of the engine involved
+        fds = []
+        for va, h, asz in owned:
+            fd = C.c_int(-1)
+            if lib.amem_vmm_export(h, C.byref(fd)) != 0:
+                break
+            fds.append(fd.value)
+        open_at_once = len(fds)
+        for fd in fds:
+            os.close(fd)
+        assert lib.amem_ipc_act_as(rank) == 0
+        for va, h, asz in owned:
+            fd, iva, ih = C.c_int(-1), C.c_uint64(), C.c_uint64()
+            assert lib.amem_vmm_export(h, C.byref(fd)) == 0
+            assert lib.amem_vmm_import(fd.value, asz, 0, C.byref(iva), C.byref(ih)) == 0
+            os.close(fd.value)
+            assert lib.amem_add_alloc_info(iva.value, asz, B.TYPE_PEER_POSIX, 0, ih.value, owner, h, None, B.CALLER_P2P_PEER) == 0
+            imports.append(iva.value)
+        assert lib.amem_ipc_act_as(-1) == 0
+
+        def bad():
+            n, buf = 0, np.empty(4096, dtype=np.uint8)
+            for i in range(N):
+                for base in (owned[i][0], imports[i]):
+                    assert lib.amem_copy_from_device(buf.ctypes.data, base + (i % 32) * 65536, 4096) == 0
+                    n += int(np.count_nonzero(buf != data[i]))
+            return n
+
+        assert bad() == 0
+        assert lib.amem_mem_pause(0, 0) == 0 and lib.amem_mem_resume(0, 0) == 0     # warm cycle: engine scratch, pinned pool
+        fds0 = _nfds()
+        for cycle in range(2):
+            assert lib.amem_mem_pause(0, 0) == 0
+            c = H.counters(lib)
+            assert (c["offload_cnt"], c["release_shadow_cnt"], c["release_local_cnt"]) == (N, N, N)
+            assert lib.amem_mem_resume(0, 0) == 0
+            c = H.counters(lib)
+            assert (c["offload_cnt"], c["release_shadow_cnt"], c["release_local_cnt"], c["paused"]) == (0, 0, 0, 0)
+            assert _nfds() == fds0 and bad() == 0
+        st = H.cycle_stats(lib)
+        measured("exported descriptors this runtime lets a process hold open: %d; %d shared regions resumed, "
+                 "pause %.0f ms, resume %.0f ms of which %.0f ms export + notify + wait" %
+                 (open_at_once, N, st["pause_ms"], st["resume_ms"], st["resume_peer_ms"]))
+        for i in range(N):
+            lib.amem_del_alloc_info(imports[i], 0, 0)
+            lib.amem_vmm_free(imports[i], owned[i][2], 0)
+            lib.amem_del_alloc_info(owned[i][0], 0, 0)
+            lib.amem_vmm_free(owned[i][0], owned[i][2], 0)
+    finally:
+        lib.amem_mem_resume(0, 0)
+        lib.amem_ipc_act_as(-1)
+        assert lib.amem_set_option(b"peer_loopback", 0) == 0
