@@ -3,6 +3,8 @@
 #include <stdio.h>
 #include <unistd.h>
 
+#include <mutex>
+
 #include "log.h"
 
 namespace amem {
@@ -194,6 +196,13 @@ hipError_t vmm_export_fd(uint64_t handle, int* fd) {
 
 hipError_t vmm_import_map(int dev, uint64_t va, size_t size, int fd, bool close_fd,
                           uint64_t* new_handle) {
+  // One import at a time per process. Several service threads of one process (one per rank it hosts)
+  // may be asked to map descriptors at the same moment; the runtime runs these calls one after the
+  // other anyway, and importing, mapping and granting access from three threads at once has failed
+  // here now and then (hipMemSetAccess on the fresh mapping: invalid argument) in a process that
+  // held several hundred other descriptors open. Importers in different processes are not affected.
+  static std::mutex one_at_a_time;
+  std::lock_guard<std::mutex> serial(one_at_a_time);
   hipMemGenericAllocationHandle_t h = nullptr;
   // hipMemMap accepts an address that already holds a mapping (measured on ROCm 7.2) and the old
   // mapping is then lost without having been unmapped: refuse here what the runtime does not.

@@ -270,6 +270,23 @@ def main():
                       "what": "amem_memPause/amem_memResume loop structure of the reference (amem_nccl.cpp:502-558, "
                               ":604-630) written with hipMemcpyAsync + sync per region on this GPU; p50 of 5 cycles"}
 
+    # The gather kernel at its full width: the default pause narrows it on purpose while it is ahead of the
+    # unmaps, which lowers its own rate and shortens the pause. Four extra cycles with the narrowing off show
+    # what the kernel does when left alone, and what the pause then costs (outside the timed region).
+    full_width = None
+    if args.config == 3 and lib.amem_get_option(b"pause_adaptive") == 1 and lib.amem_get_option(b"pause_path") in (2, 3):
+        assert lib.amem_set_option(b"pause_adaptive", 0) == 0
+        fp_s, _, fst, _ = run_cycles(1, 4)
+        assert lib.amem_set_option(b"pause_adaptive", 1) == 0
+        fk2 = statistics.median(s_["k2_ms"] for s_ in fst)
+        fkb = statistics.mean(s_["kernel_bytes"] for s_ in fst)
+        full_width = {"device_ms_per_pause": round(fk2, 3), "GBps": round(fkb / fk2 / 1e6, 2),
+                      "frac_of_measured_d2h": round(fkb / fk2 / 1e6 / d2h.value, 4),
+                      "p50_pause_s": round(statistics.median(fp_s), 4),
+                      "unmap_us_each_p50": round(statistics.median(s_["pause_unmap_ms"] for s_ in fst) * 1e3 / len(fp.sizes), 1),
+                      "what": "the same kernel with every launch 8 workgroups wide (pause_adaptive=0), p50 of 4 cycles after "
+                              "the timed ones: the kernel itself is faster, each unmap beside it costs more, the pause is longer"}
+
     # The pack and unpack kernels on their own against the HBM roofline: the footprint's non-zero runs
     # gathered into one device buffer and scattered back (S read + S written each way), through the C ABI.
     hbm_kernels = None
@@ -394,6 +411,7 @@ def main():
                 "device_ms_per_resume": round(k3_ms, 3), "GBps": round(parked / k3_ms / 1e6, 2) if k3_ms else None,
                 "frac_of_measured_h2d": round(parked / k3_ms / 1e6 / h2d.value, 4) if k3_ms else None,
                 "frac_of_pcie_gen5_x16": round(parked / k3_ms / 1e6 / PCIE_GEN5_X16, 4) if k3_ms else None},
+            "gather_at_full_width": full_width,
             "what": "device time from HIP events on the launch stream (first launch to last, the sum over a leg's launches); "
                     "these two kernels are over 99 % of the GPU time of a cycle, the scan kernel of `roofline` under 1 %"},
         "unmap": {"regions": len(fp.sizes), "us_each_p50": round(statistics.median(s["pause_unmap_ms"] for s in stats)

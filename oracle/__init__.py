@@ -64,6 +64,7 @@ def load():
         "oracle_vmm_export": (i, [u64, P(i)]),
         "oracle_vmm_import": (i, [i, u64, P(u64), P(u64)]),
         "oracle_vmm_live_bytes": (u64, []),
+        "oracle_vmm_reset": (None, []),
         "oracle_vmm_handle_of": (u64, [u64]),
         "oracle_vmm_retain": (u64, [u64]),
         "oracle_reset": (None, []),

@@ -158,6 +158,19 @@ API uint64_t oracle_vmm_handle_of(uint64_t va) {
   return h;
 }
 
+/* Test hygiene: drop everything the host-memory stand-in still holds (mappings go back to nothing,
+   physical objects are closed), so that a test that did not free its regions one by one leaves no
+   descriptors or memory behind for the next one. Reservations of regions that were paused at that
+   moment (address space only, no memory) are left to the process's end. */
+API void oracle_vmm_reset(void) {
+  pthread_mutex_lock(&g_vmm_mtx);
+  for (size_t i = 0; i < g_nmaps; ++i) munmap((void*)(uintptr_t)g_maps[i].va, g_maps[i].size);
+  g_nmaps = 0;
+  for (size_t i = 0; i < g_nphys; ++i)
+    if (g_phys[i].live) { close(g_phys[i].fd); g_phys[i].live = 0; }
+  pthread_mutex_unlock(&g_vmm_mtx);
+}
+
 API uint64_t oracle_vmm_live_bytes(void) {
   uint64_t n = 0;
   pthread_mutex_lock(&g_vmm_mtx);

@@ -59,6 +59,7 @@ int oracle_vmm_free(uint64_t va, uint64_t alloc_size, uint64_t handle);
 int oracle_vmm_export(uint64_t handle, int* fd);
 int oracle_vmm_import(int fd, uint64_t size, uint64_t* va, uint64_t* handle);
 uint64_t oracle_vmm_live_bytes(void);   /* bytes of physical memory (memfds) still referenced */
+void oracle_vmm_reset(void);            /* test hygiene: unmap and close everything the stand-in still holds */
 uint64_t oracle_vmm_handle_of(uint64_t va);
 uint64_t oracle_vmm_retain(uint64_t va);   /* one more reference, as cuMemRetainAllocationHandle takes */
 

@@ -27,6 +27,30 @@ def measured():
     return _MEASURED.append
 
 
+def _fd_kinds():
+    kinds = {}
+    for f in os.listdir("/proc/self/fd"):
+        try:
+            t = os.readlink("/proc/self/fd/" + f)
+        except OSError:
+            continue
+        k = t.split(":")[0] if not t.startswith("/") else ("/dmabuf" if t.startswith("/dmabuf") else t)
+        kinds[k] = kinds.get(k, 0) + 1
+    return kinds
+
+
+@pytest.fixture(autouse=True)
+def _descriptor_growth(request):
+    """Notes every test after which this process holds noticeably more open descriptors than before it."""
+    before = len(os.listdir("/proc/self/fd"))
+    yield
+    after = len(os.listdir("/proc/self/fd"))
+    if after - before > 16:
+        top = sorted(_fd_kinds().items(), key=lambda kv: -kv[1])[:4]
+        _MEASURED.append("descriptors: %s left %d more open (%d -> %d); most common now: %s" %
+                         (request.node.name, after - before, before, after, top))
+
+
 def pytest_terminal_summary(terminalreporter):
     if _MEASURED:
         terminalreporter.section("measured")
@@ -76,6 +100,7 @@ def fresh_orc(orc):
     orc.oracle_reset()
     yield orc
     orc.oracle_reset()
+    orc.oracle_vmm_reset()      # regions a test left in the oracle's host-memory stand-in (one memfd each)
 
 
 @pytest.fixture(scope="session")
