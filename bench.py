@@ -36,6 +36,8 @@ import statistics
 import sys
 import time
 
+import numpy as np
+
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
@@ -123,7 +125,37 @@ def numa_placement(lib, slab_addr):
     return out
 
 
-def time_config(lib, B, H, fp, warmup, steps, d2h, h2d):
+def suballocation_kernels(lib, B, regs, pg):
+    """Configuration 4's 100,000 sub-allocations as a descriptor list: gathered out of their granules into one
+    device buffer and scattered back by the pack/unpack kernel (device memory on both sides), through the C ABI."""
+    g = pg.GRANULE
+    n = len(pg.starts)
+    sizes = pg.sub.sizes.astype(np.uint64)
+    descs = np.empty((n, 3), dtype=np.uint64)
+    descs[:, 0] = regs.va[(pg.starts // g).astype(np.int64)] + (pg.starts % g).astype(np.uint64)
+    descs[:, 1] = np.concatenate([[0], np.cumsum(sizes)[:-1]]).astype(np.uint64)
+    descs[:, 2] = sizes
+    S = int(sizes.sum())
+    sva, sh, sasz = C.c_uint64(), C.c_uint64(), C.c_uint64()
+    if lib.amem_vmm_alloc(S, 0, C.byref(sva), C.byref(sh), C.byref(sasz)) != 0:
+        return None
+    dptr = descs.ctypes.data_as(C.POINTER(B.CopyDesc))
+    gms, sms, ms = [], [], C.c_float()
+    for _ in range(4):
+        assert lib.amem_gather_pack(dptr, n, C.c_void_p(sva.value), S, 0, C.byref(ms)) == 0
+        gms.append(ms.value)
+        assert lib.amem_scatter_unpack(dptr, n, C.c_void_p(sva.value), S, 0, C.byref(ms)) == 0
+        sms.append(ms.value)
+    lib.amem_vmm_free(sva.value, sasz.value, sh.value)
+    gm, sm = statistics.median(gms[1:]), statistics.median(sms[1:])
+    return {"descriptors": n, "packed_bytes": S,
+            "gather_pack": {"ms": round(gm, 3), "GBps": round(2 * S / gm / 1e6, 1), "frac_of_hbm_peak": round(2 * S / gm / 1e6 / HBM_PEAK_GBPS, 4)},
+            "scatter_unpack": {"ms": round(sm, 3), "GBps": round(2 * S / sm / 1e6, 1), "frac_of_hbm_peak": round(2 * S / sm / 1e6 / HBM_PEAK_GBPS, 4)},
+            "what": "move_pieces_hbm over one descriptor per sub-allocation (4-64 KiB each, 2*S bytes per launch: S read + S "
+                    "written), p50 of 3 launches after a warm one; the granules' bytes are checked afterwards with the rest"}
+
+
+def time_config(lib, B, H, fp, warmup, steps, d2h, h2d, extra=None):
     """One footprint through `warmup` untimed and `steps` timed pause/resume cycles, with the correctness gate."""
     regs = H.Regions(lib, fp)
     F = int(regs.alloc.sum())
@@ -140,6 +172,7 @@ def time_config(lib, B, H, fp, warmup, steps, d2h, h2d):
         assert rc1 == 0 and rc2 == 0, (rc1, rc2)
         if step >= warmup:
             pause_s.append(t1 - t0); resume_s.append(t2 - t1); stats.append(H.cycle_stats(lib))
+    more = extra(regs, fp) if extra else None
     bad = regs.mismatched_bytes()
     tdiff = [d for d in H.compare_tables(table_before, regs.table()) if d[1] != "handle_gen"]
     ok = bad == 0 and bool((regs.va == va_before).all()) and not tdiff
@@ -155,7 +188,7 @@ def time_config(lib, B, H, fp, warmup, steps, d2h, h2d):
             "resume_leg_frac_of_link": round(parked / pr / 1e9 / h2d, 4),
             "pause_us_per_region": round(pp * 1e6 / n, 1), "resume_us_per_region": round(pr * 1e6 / n, 1),
             "unmap_us_each_p50": round(statistics.median(s["pause_unmap_ms"] for s in stats) * 1e3 / n, 1),
-            "bit_exact": ok}
+            "bit_exact": ok, **({"suballocation_kernels": more} if more else {})}
 
 
 def main():
@@ -441,7 +474,8 @@ def main():
         for name, make in (("config_1", lambda: Footprint(1, 0, threads=host_threads)),
                            ("config_2", lambda: Footprint(2, 1, threads=host_threads)),
                            ("config_4", lambda: PackedGranules(3, 100000, threads=host_threads))):
-            others[name] = time_config(lib, B, H, make(), 1, 5, d2h.value, h2d.value)
+            extra = (lambda r, f: suballocation_kernels(lib, B, r, f)) if name == "config_4" else None
+            others[name] = time_config(lib, B, H, make(), 1, 5, d2h.value, h2d.value, extra)
             ok = ok and others[name]["bit_exact"]
         others["what"] = ("the other single-process configurations of the benchmark, 5 timed cycles each after a warm one, "
                           "1 % of chunks rewritten between cycles where the footprint has a generator for it: config 1 = 64 "

@@ -178,7 +178,7 @@ def test_pack_unpack_match_oracle(gpu, orc, host_side):
 
 
 @pytest.mark.parametrize("count", [2000, 100000])
-def test_fragmented_descriptor_list_round_trip(gpu, orc, count):
+def test_fragmented_descriptor_list_round_trip(gpu, orc, count, measured):
     """benchmark configuration 4 (100,000 sub-allocations of 4-64 KiB bump-packed into 2 MiB granules, seed 3;
     also at 1/50 scale): gathered into contiguous staging and scattered back into fresh memory."""
     fp = Footprint(4, 3, max_regions=count, threads=16)
@@ -207,6 +207,7 @@ def test_fragmented_descriptor_list_round_trip(gpu, orc, count):
     garr[:, 2] = sizes
     ms = C.c_float()
     assert gpu.amem_gather_pack(garr.ctypes.data_as(C.POINTER(B.CopyDesc)), len(sizes), stage.va, packed, 0, C.byref(ms)) == 0
+    gather_ms = ms.value
     live = np.zeros(total, dtype=bool)
     idx = np.concatenate([np.arange(a, a + n) for a, n in zip(starts[:4000], sizes[:4000])])   # spot-check layout
     got = stage.get(packed)
@@ -219,6 +220,10 @@ def test_fragmented_descriptor_list_round_trip(gpu, orc, count):
     assert gpu.amem_scatter_unpack(sarr.ctypes.data_as(C.POINTER(B.CopyDesc)), len(sizes), stage.va, packed, 0, C.byref(ms)) == 0
     back = dst.get(total)
     assert np.array_equal(back[live], host[live]) and (back[~live] == 0x77).all()
+    if count == 100000:
+        measured("config 4's %d sub-allocations as one descriptor each, %.2f GB packed: gather %.2f ms = %.2f TB/s, scatter %.2f ms "
+                 "= %.2f TB/s (S read + S written; first launches)" % (len(sizes), packed / 1e9, gather_ms, 2 * packed / gather_ms / 1e9,
+                                                                      ms.value, 2 * packed / ms.value / 1e9))
     src.free(); dst.free(); stage.free()
 
 
