@@ -72,14 +72,14 @@ int main(int argc, char** argv) {
       std::this_thread::yield();
     }
   });
-  for (int cycle = 0; cycle < 8; ++cycle) {
+  for (int cycle = 0; cycle < 6; ++cycle) {
     EXPECT(amem_mem_pause(0, 0) == 0);
     EXPECT(amem_check_paused(0) == 1);
     EXPECT(amem_mem_resume(0, 0) == 0);
     amem_cycle_stats st;
     amem_get_cycle_stats(&st);
     EXPECT(st.verify_mismatch == 0);
-    add_buffers(6 << (cycle / 2));                          // more regions, more chunks: the engine's tables regrow
+    add_buffers(4 << (cycle / 2));                          // more regions, more chunks: the engine's tables regrow
     usleep(2000);
   }
   stop.store(true);
@@ -89,6 +89,6 @@ int main(int argc, char** argv) {
   for (void* p : bufs) EXPECT(cumem_free(p) == 0);
   EXPECT(plain_free(served) == 0);
   EXPECT(registered() == 0 && amem_region_count(0) == 0);
-  printf("hook race done: %ld errors, %ld exports beside 8 cycles, %zu buffers\n", g_errors.load(), exports.load(), bufs.size());
+  printf("hook race done: %ld errors, %ld exports beside 6 cycles, %zu buffers\n", g_errors.load(), exports.load(), bufs.size());
   return g_errors.load() ? 1 : 0;
 }
