@@ -113,7 +113,11 @@ int amem_add_peer_info(uint64_t src_va, uint64_t peer_va, int peer_dev);
 
 /* Owner-side half of an import: find the local region that `src_handle` backs and
  * record the importer's VA. Replaces amem_registerPeerInfo, amem_nccl.cpp:297-329.
- * Runs on the IPC service thread when an importer registers. 0 ok, 1 not found. */
+ * Runs on the IPC service thread when an importer registers. 0 ok, 1 not found.
+ * Extension: a value that is no handle of this process is also looked up as the address of a
+ * local region. An importer that cannot know the owner's current handle value (it changes with
+ * every resume) may name the region by the owner's address, which never changes; the allocator
+ * hook for an unpatched RCCL does. */
 int amem_register_peer_info(uint64_t src_handle, uint64_t peer_va, int peer_dev);
 
 /* Importer-side half of a resume: import `shared_fd`, map it at the region's original VA,

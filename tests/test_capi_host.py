@@ -120,6 +120,26 @@ def test_registry_matches_oracle_call_for_call(fresh, fresh_orc):
     assert lib.amem_check_paused(0) == orc.oracle_check_paused(0) == 0
 
 
+def test_importer_may_name_a_region_by_the_owners_address(fresh):
+    """amem_registerPeerInfo finds the owner's region by handle (amem_nccl.cpp:303-316). Here a value
+    that is no handle of the process is looked up as a local region's address as well: a handle value
+    noted at export time is dead after the owner's next resume, the address is not. A value that is
+    neither is still refused."""
+    lib = fresh
+    va, h = 0x7e0000200000, 0xabc0
+    assert lib.amem_add_alloc_info(va, 2 * MiB, B.TYPE_LOCAL, 0, h, -1, 0, None, B.CALLER_P2P) == 0
+    assert lib.amem_register_peer_info(h, 0x7d0000000000, 3) == 0           # by handle, as the reference does
+    assert lib.amem_register_peer_info(va, 0x7d0000400000, 5) == 0          # by the owner's address
+    t = H.region_table(lib, 0)[va]
+    assert t["has_peer"] == 1 and t["peers"][3] == 0x7d0000000000 and t["peers"][5] == 0x7d0000400000
+    assert lib.amem_register_peer_info(va + 4096, 0x7d0000800000, 6) == 1   # not the start of a region
+    assert lib.amem_register_peer_info(0x1234, 0x7d0000800000, 6) == 1      # neither handle nor address
+    imp = 0x7e0000800000                                                    # an import whose owner cannot be reached is dropped
+    assert lib.amem_add_alloc_info(imp, 2 * MiB, B.TYPE_PEER_POSIX, 0, 0xdef0, -1, h, None, B.CALLER_P2P_PEER) != 0
+    assert lib.amem_register_peer_info(imp, 0x7d0000c00000, 2) == 1
+    assert lib.amem_del_alloc_info(va, h, 0) == 0
+
+
 def test_region_order_and_find(fresh):
     lib = fresh
     vas = [0x7f0030000000, 0x7f0010000000, 0x7f0020000000]
