@@ -124,6 +124,43 @@ def test_repeated_cycles_with_writes_between(eng):
     regs.free()
 
 
+def test_a_hundred_cycles_leave_nothing_behind(eng, measured):
+    """A serving process pauses and resumes for as long as it lives (the reference's RL loop does it every
+    step, README.md:21-25). 100 cycles of a 1 GiB training-rank footprint with writes in between: device
+    memory in use, pinned host memory held, open descriptors and the process's own resident memory are the
+    same after the last cycle as after the second, every cycle is verified chunk by chunk, and the bytes
+    are compared with regenerated ones at the end."""
+    import resource
+    lib = eng
+    fp = Footprint(3, 2, byte_budget=1 << 30, threads=16)
+    regs = H.Regions(lib, fp)
+    assert lib.amem_set_option(b"verify", 1) == 0
+    nfds = lambda: len(os.listdir("/proc/self/fd"))
+    rss_kib = lambda: int(open("/proc/self/statm").read().split()[1]) * resource.getpagesize() // 1024
+    marks = []
+    for cycle in range(100):
+        regs.write_chunks(fp.mutate(cycle))
+        assert lib.amem_mem_pause(0, 0) == 0
+        assert lib.amem_mem_resume(0, 0) == 0
+        st = H.cycle_stats(lib)
+        assert st["verify_mismatch"] == 0 and st["zero_chunks"] == fp.zero_chunks()
+        if cycle in (1, 99):
+            marks.append((H.mem_free(lib), st["slab_bytes"], nfds(), rss_kib()))
+    (free_a, slab_a, fd_a, rss_a), (free_b, slab_b, fd_b, rss_b) = marks
+    assert abs(free_a - free_b) <= 8 * MiB, (free_a, free_b)          # no device memory lost or kept
+    assert slab_a == slab_b and fd_a == fd_b                          # the pinned pool is reused, nothing stays open
+    assert rss_b - rss_a <= 64 * 1024, (rss_a, rss_b)                 # KiB: the host side does not grow either
+    assert regs.mismatched_bytes() == 0
+    c = H.counters(lib)
+    assert c["pause_cnt"] == c["resume_cnt"] == 100 and (c["offload_cnt"], c["release_local_cnt"], c["release_shadow_cnt"]) == (0, 0, 0)
+    tab = regs.table()
+    assert all(t["handle_gen"] == 101 for t in tab.values())          # a new physical handle per cycle at every address
+    measured("100 cycles of 1 GiB: device memory free %+.1f MiB, pinned pool %d MiB both times, descriptors %d both times, "
+             "resident host memory %+.1f MiB between the 2nd and the 100th cycle" %
+             ((free_b - free_a) / MiB, slab_b >> 20, fd_b, (rss_b - rss_a) / 1024))
+    regs.free()
+
+
 @pytest.mark.parametrize("opts", [{"zero_elide": 0}, {"scratch_on_host": 1}, {"scratch_on_host": 1, "pause_path": 1}, {"pause_path": 0, "dma_min_bytes": 128 << 10},
                                   {"staging_bytes": 8 << 20}, {"resume_batch_bytes": 1},
                                   {"staging_bytes": 1 << 20, "resume_batch_bytes": 1 << 40},
