@@ -298,8 +298,9 @@ hipError_t launch_move(bool scatter, const CopyDesc* d_descs, const uint64_t* d_
 // Scan without allocation. The scan needs device memory beyond its inputs and outputs: the
 // segment table, the chunk prefix, and the flag and checksum arrays the kernel writes before
 // they are copied to the host. The ordinary path keeps those in growable hipMalloc buffers;
-// callers that may not allocate (code under graph capture, tight serving loops, harnesses that
-// forbid it) use this fixed array instead. Every GPU the library runs on holds its own copy of
+// callers that may not allocate (tight serving loops, harnesses that forbid it) use this fixed
+// array instead; the call synchronises its stream, so it belongs outside any stream capture.
+// Every GPU the library runs on holds its own copy of
 // the array, at its own address, until the process ends.
 // ------------------------------------------------------------------------------------
 
