@@ -57,7 +57,8 @@ class CycleStats(C.Structure):
         "k1_launches", "k2_launches", "k3_launches", "footprint_bytes", "parked_bytes", "zero_chunks",
         "total_chunks", "local_regions", "peer_regions", "dma_bytes", "kernel_bytes", "slab_bytes",
         "verify_mismatch")] + [(n, C.c_double) for n in (
-        "pause_pool_ms", "pause_scratch_ms", "pause_sync_ms", "resume_scratch_ms")] + [("resume_dma_bytes", C.c_uint64), ("pause_narrow_launches", C.c_uint64)]
+        "pause_pool_ms", "pause_scratch_ms", "pause_sync_ms", "resume_scratch_ms")] + [("resume_dma_bytes", C.c_uint64), ("pause_narrow_launches", C.c_uint64),
+                                                                         ("resume_plan_ms", C.c_double)]
 
     def as_dict(self):
         return {k: getattr(self, k) for k, _ in self._fields_}

@@ -1089,6 +1089,7 @@ int Engine::resume(Ctx& c, bool* incomplete) {
   auto t0 = Clock::now();
   stats_.resume_ms = stats_.resume_map_ms = stats_.resume_copy_ms = stats_.resume_peer_ms = 0;
   stats_.k3_ms = 0; stats_.k3_launches = 0; stats_.verify_mismatch = 0; stats_.resume_dma_bytes = 0;
+  stats_.resume_plan_ms = 0;
   (void)take_scratch_alloc_ms();
   auto& table = c.allocTable[dev_];
 
@@ -1105,10 +1106,16 @@ int Engine::resume(Ctx& c, bool* incomplete) {
   // Scatter list: per region, its parked runs and its zero runs.
   struct Item { Region* r; uint64_t va; uint32_t d0, d1; uint64_t bytes; uint32_t m0, m1; };
   std::vector<Item> items;
-  std::vector<CopyDesc> scatter;
+  items.reserve(table.size());
+  // The lists are members so that their memory is kept from cycle to cycle: tens of thousands of
+  // descriptors built into fresh vectors cost the resume 2 ms of allocation and first touches.
+  std::vector<CopyDesc>& scatter = scatter_descs_;
+  scatter.clear();
   // Runs at least resume_dma_min_bytes long (0 = none) come back by hipMemcpyAsync on the second
   // stream, next to the scatter kernel on the first; `dma` holds them, an item's are [m0, m1).
-  std::vector<CopyDesc> dma;
+  std::vector<CopyDesc>& dma = dma_descs_;
+  dma.clear();
+  std::vector<CopyDesc>& zeros = zero_descs_;
   const uint64_t dma_min = ref_mode_ ? 0 : (uint64_t)options().resume_dma_min_bytes;
   const uint8_t* flags = parked_flags_.data();
   const uint64_t slab_bytes = pool_->slab_bytes();
@@ -1122,7 +1129,7 @@ int Engine::resume(Ctx& c, bool* incomplete) {
     if (r.state != AMEM_STATE_HOLE || from_peer(r.type)) continue;
     Item im = {&r, p.va, (uint32_t)scatter.size(), 0, p.size, (uint32_t)dma.size(), 0};
     uint64_t cursor = p.parked_off;
-    std::vector<CopyDesc> zeros;
+    zeros.clear();
     emit_runs(flags + p.first_chunk, p.va, p.size, elide || p.skip, &cursor, slab_bytes, &scatter, &zeros, nullptr);
     if (dma_min) {
       size_t keep = im.d0;
@@ -1166,6 +1173,7 @@ int Engine::resume(Ctx& c, bool* incomplete) {
   uint64_t exportSz = 0;
   size_t ev = 8;
   std::vector<std::pair<hipEvent_t, hipEvent_t>> timed;
+  stats_.resume_plan_ms = ms_since(t0);
   auto tc = Clock::now();
   const uint64_t batch_bytes = (uint64_t)std::max<int64_t>(options().resume_batch_bytes, 1);
   size_t i = 0;

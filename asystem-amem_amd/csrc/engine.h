@@ -143,6 +143,7 @@ class Engine {
   // state carried from pause to resume
   std::vector<ParkedRegion> parked_;
   std::vector<CopyDesc> gather_descs_;
+  std::vector<CopyDesc> scatter_descs_, dma_descs_, zero_descs_;  // resume's lists; kept for their capacity
   std::vector<ScanSeg> segs_;
   uint64_t nchunks_ = 0;
   uint64_t parked_total_ = 0;

@@ -43,7 +43,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
 PHASES = ("pause_sync_ms", "pause_scan_ms", "pause_plan_ms", "pause_pool_ms", "pause_scratch_ms", "pause_copy_ms",
-          "pause_unmap_ms", "resume_map_ms", "resume_copy_ms", "resume_peer_ms", "resume_scratch_ms",
+          "pause_unmap_ms", "resume_plan_ms", "resume_map_ms", "resume_copy_ms", "resume_peer_ms", "resume_scratch_ms",
           "k1_ms", "k2_ms", "k3_ms")
 
 

@@ -265,6 +265,7 @@ typedef struct amem_cycle_stats {
   double resume_scratch_ms; /* of resume_ms: allocating or growing the engine's own tables and events */
   uint64_t resume_dma_bytes; /* of parked_bytes, how much the resume brought back by hipMemcpyAsync */
   uint64_t pause_narrow_launches; /* of k2_launches, how many "pause_adaptive" issued with fewer workgroups */
+  double resume_plan_ms;    /* of resume_ms: host work before the first region is mapped (scatter list, table upload) */
 } amem_cycle_stats;
 void amem_get_cycle_stats(amem_cycle_stats* out);
 
