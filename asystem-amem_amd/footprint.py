@@ -82,6 +82,23 @@ class Footprint:
         self.gen = np.zeros(max(self.nchunks, 1), dtype=np.uint32)
         self.total_bytes = int(self.sizes.sum())
 
+    @classmethod
+    def with_sizes(cls, sizes, seed, zero_pct=30, threads=8):
+        """A footprint of the given region sizes (bytes, multiples of 16) instead of a configuration's
+        draw list; zero mask and contents come from the same generator, keyed by seed and chunk number."""
+        self = cls.__new__(cls)
+        self.cfg, self.seed, self.threads = 0, seed, threads
+        self.sizes = np.array(sizes, dtype=np.uint64)
+        chunks = (self.sizes + np.uint64(CHUNK - 1)) // np.uint64(CHUNK)
+        self.first_chunk = np.concatenate([[0], np.cumsum(chunks)]).astype(np.uint64)
+        self.nchunks = int(self.first_chunk[-1])
+        self.mask = np.zeros(max(self.nchunks, 1), dtype=np.uint8)
+        if zero_pct:
+            lib().amem_fp_zero_mask(seed, self.nchunks, zero_pct, _ptr(self.mask))
+        self.gen = np.zeros(max(self.nchunks, 1), dtype=np.uint32)
+        self.total_bytes = int(self.sizes.sum())
+        return self
+
     def region_bytes(self, i, out=None):
         """Bytes of region i as a uint8 array."""
         n = int(self.sizes[i])

@@ -382,6 +382,43 @@ def test_config3_as_worded_all_2560_regions(eng, measured):
     lib.amem_pool_trim()                                      # 33 GB of pinned host memory go back
 
 
+def test_regions_larger_than_4_GiB(eng, measured):
+    """Single regions beyond what 32 bits can count: 5 GiB + 2 MiB (81,952 chunks and 15 slabs' worth of
+    parked bytes in one region), exactly 4 GiB, and a small one between them. Two verified cycles with
+    writes in between; all bytes are read back and compared with regenerated ones, addresses and table
+    fields stay, the memory is really given back while paused."""
+    lib = eng
+    sizes = [5 * GiB + 2 * MiB, 2 * MiB, 4 * GiB]
+    if H.mem_free(lib) < sum(sizes) + 4 * GiB:
+        pytest.skip("needs %d GiB of free device memory" % ((sum(sizes) >> 30) + 4))
+    fp = Footprint.with_sizes(sizes, seed=44, zero_pct=30, threads=16)
+    regs = H.Regions(lib, fp)
+    assert [int(a) for a in regs.alloc] == sizes
+    before, va_before = regs.table(), regs.va.copy()
+    assert lib.amem_set_option(b"verify", 1) == 0
+    times = []
+    for cycle in range(1, 3):
+        regs.write_chunks(fp.mutate(cycle, fraction=0.002))
+        free1 = H.mem_free(lib)
+        assert lib.amem_mem_pause(0, 0) == 0
+        if cycle > 1:
+            assert H.mem_free(lib) - free1 >= fp.total_bytes - 64 * MiB
+        st = H.cycle_stats(lib)
+        assert st["local_regions"] == 3 and st["footprint_bytes"] == sum(sizes)
+        assert st["total_chunks"] == fp.nchunks and st["zero_chunks"] == fp.zero_chunks()
+        assert st["parked_bytes"] == (fp.nchunks - fp.zero_chunks()) * CHUNK
+        assert lib.amem_mem_resume(0, 0) == 0
+        st = H.cycle_stats(lib)
+        assert st["verify_mismatch"] == 0
+        times.append((st["pause_ms"], st["resume_ms"]))
+    assert (regs.va == va_before).all()
+    assert regs.mismatched_bytes() == 0
+    assert [d for d in H.compare_tables(before, regs.table()) if d[1] != "handle_gen"] == []
+    measured("regions of 5 GiB + 2 MiB, 2 MiB and 4 GiB (%.2f GB parked): pause / resume ms %s" %
+             (st["parked_bytes"] / 1e9, ", ".join("%.0f / %.0f" % t for t in times)))
+    regs.free()
+
+
 def test_config1_cycle_beside_the_oracle(eng, fresh_orc):
     """benchmark configuration 1 (64 regions of 2 MiB x U{1..16}, seed 0, no zero chunks): the engine on
     the GPU and the oracle in host memory make the same calls; bytes, table, counters and per-region
